@@ -99,7 +99,11 @@ def read_config_json(model_dir: str) -> Dict[str, Any]:
 
 def architecture_name(raw: Dict[str, Any]) -> str:
     """`architectures[0]`, the key of the model registry
-    (reference src/models/config.cpp:12-14 stores it; it has no registry)."""
+    (reference src/models/config.cpp:12-14 stores it; it has no registry); a config.json
+    that names its one architecture as a string under `architecture` is read too."""
+    one = raw.get("architecture")
+    if "architectures" not in raw and isinstance(one, str) and one:
+        return one
     arch = raw.get("architectures")
     if not isinstance(arch, list) or not arch or not isinstance(arch[0], str):
         raise ConfigError("config.json: key 'architectures' must be a non-empty list of names")

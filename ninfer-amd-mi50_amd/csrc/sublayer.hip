@@ -1,0 +1,172 @@
+// Row-wise kernels around a sublayer whose norm sits on its output:
+//
+//   short_conv     h_t + sum_j w[:, j] h_(t - taps + 1 + j): a causal convolution over the
+//                  rows of each request, channel by channel, added to its input. The last
+//                  taps - 1 inputs of a request are per-request state (32-bit), so a request
+//                  may be cut into steps anywhere; before a request's start they are zero.
+//   norm_add       x += y rsqrt(mean(y^2) + eps) g, g one number or one per channel.
+//   gated_rmsnorm  out = o rsqrt(mean(o^2) + eps) w sigmoid(g), the norm over the whole row.
+//
+// All sums are 32-bit and their order depends on the row alone (taps ascending; the block
+// reduction's order depends on the width), never on how a request was cut or on the batch.
+#include "common.h"
+
+namespace ninfer {
+
+// out[t, c] for all rows. Inputs before the step's first row of a request come from the
+// request's state: state[slot][i * H + c] is the input at the request's position
+// pos0 - (taps - 1) + i. With `update` (steps in which every request brings one row) the
+// thread also shifts the state; otherwise short_conv_state_kernel does so afterwards.
+template <typename T>
+__global__ void short_conv_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                  float* __restrict__ state, int64_t state_stride,
+                                  T* __restrict__ out, const int* __restrict__ row_seq,
+                                  const int* __restrict__ seq_row_start,
+                                  const int* __restrict__ seq_slots, int H, int taps, int update) {
+  const int t = blockIdx.x;
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= H) return;
+  const int s = row_seq[t];
+  const int r0 = seq_row_start[s];
+  const int i = t - r0;
+  float* st = state + (int64_t)seq_slots[s] * state_stride;
+  const float* wc = w + (int64_t)c * taps;
+  const float cur = x[(int64_t)t * H + c];
+  float acc = 0.f;
+  for (int j = 0; j < taps; ++j) {
+    const int src = i - (taps - 1 - j);
+    const float v = src >= 0 ? x[(int64_t)(r0 + src) * H + c] : st[(int64_t)(taps - 1 + src) * H + c];
+    acc = fmaf(wc[j], v, acc);
+  }
+  out[(int64_t)t * H + c] = from_f32<T>(cur + acc);
+  if (update) {   // this row is the request's only one: the state moves on by one input
+    for (int k = 0; k + 2 < taps; ++k) st[(int64_t)k * H + c] = st[(int64_t)(k + 1) * H + c];
+    if (taps > 1) st[(int64_t)(taps - 2) * H + c] = cur;
+  }
+}
+
+// state <- the last taps - 1 inputs of each request after this step's n rows. Entry k is the
+// input at index n - (taps - 1) + k of the step's rows; a negative index is the old entry
+// k + n, which lies above k, so ascending k never reads what it has written.
+__global__ void short_conv_state_kernel(const float* __restrict__ x, float* __restrict__ state,
+                                        int64_t state_stride,
+                                        const int* __restrict__ seq_row_start,
+                                        const int* __restrict__ seq_slots, int H, int taps) {
+  const int s = blockIdx.x;
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= H) return;
+  const int r0 = seq_row_start[s];
+  const int n = seq_row_start[s + 1] - r0;
+  float* st = state + (int64_t)seq_slots[s] * state_stride;
+  for (int k = 0; k < taps - 1; ++k) {
+    const int p = n - (taps - 1) + k;
+    st[(int64_t)k * H + c] = p >= 0 ? x[(int64_t)(r0 + p) * H + c] : st[(int64_t)(k + n) * H + c];
+  }
+}
+
+template <typename T>
+__global__ void norm_add_kernel(float* __restrict__ x, const T* __restrict__ y,
+                                const float* __restrict__ gain, int gain_n, int H, float eps) {
+  __shared__ float red[16];
+  const int64_t r = blockIdx.x;
+  const T* yr = y + r * H;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    const float v = to_f32(yr[i]);
+    ss = fmaf(v, v, ss);
+  }
+  ss = block_sum(ss, red);
+  const float inv = 1.f / sqrtf(ss / (float)H + eps);
+  float* xr = x + r * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    const float g = gain[gain_n == 1 ? 0 : i];
+    xr[i] += to_f32(yr[i]) * inv * g;
+  }
+}
+
+template <typename T>
+__global__ void gated_rmsnorm_kernel(const float* __restrict__ o, const T* __restrict__ gate,
+                                     int gate_stride, const float* __restrict__ w,
+                                     T* __restrict__ out, int N, float eps) {
+  __shared__ float red[16];
+  const int64_t r = blockIdx.x;
+  const float* orow = o + r * N;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < N; i += blockDim.x) ss = fmaf(orow[i], orow[i], ss);
+  ss = block_sum(ss, red);
+  const float inv = 1.f / sqrtf(ss / (float)N + eps);
+  const T* g = gate + r * gate_stride;
+  for (int i = threadIdx.x; i < N; i += blockDim.x) {
+    const float sg = 1.f / (1.f + expf(-to_f32(g[i])));
+    out[r * N + i] = from_f32<T>(orow[i] * inv * w[i] * sg);
+  }
+}
+
+static int row_block(int H) {
+  int b = (H + 63) / 64 * 64;
+  return b > 256 ? 256 : b;
+}
+
+}  // namespace ninfer
+
+using namespace ninfer;
+
+extern "C" int ninfer_short_conv(const float* x, const float* w, float* state,
+                                 long long state_stride, void* out, const int* row_seq,
+                                 const int* seq_row_start, const int* seq_slots, int T, int S,
+                                 int H, int taps, int all_single, int dtype, hipStream_t stream) {
+  NINFER_REQUIRE(T > 0 && S > 0 && H > 0, "short_conv: T=%d S=%d H=%d must be positive", T, S, H);
+  NINFER_REQUIRE(taps >= 1, "short_conv: %d taps", taps);
+  NINFER_REQUIRE(state_stride >= (long long)(taps - 1) * H,
+                 "short_conv: a request's state of %lld floats holds no %d x %d inputs",
+                 state_stride, taps - 1, H);
+  NINFER_REQUIRE(dtype == kF32 || dtype == kBF16, "short_conv: unknown dtype %d", dtype);
+  const int block = row_block(H);
+  const dim3 grid(T, (H + block - 1) / block);
+  if (dtype == kF32)
+    short_conv_kernel<float><<<grid, block, 0, stream>>>(x, w, state, state_stride, (float*)out,
+                                                         row_seq, seq_row_start, seq_slots, H,
+                                                         taps, all_single);
+  else
+    short_conv_kernel<bf16><<<grid, block, 0, stream>>>(x, w, state, state_stride, (bf16*)out,
+                                                        row_seq, seq_row_start, seq_slots, H, taps,
+                                                        all_single);
+  NINFER_LAUNCH_CHECK();
+  if (!all_single && taps > 1) {
+    short_conv_state_kernel<<<dim3(S, (H + block - 1) / block), block, 0, stream>>>(
+        x, state, state_stride, seq_row_start, seq_slots, H, taps);
+    NINFER_LAUNCH_CHECK();
+  }
+  return 0;
+}
+
+extern "C" int ninfer_norm_add(float* x, const void* y, const float* gain, int gain_n, int T, int H,
+                               float eps, int dtype, hipStream_t stream) {
+  NINFER_REQUIRE(T > 0 && H > 0, "norm_add: T=%d H=%d must be positive", T, H);
+  NINFER_REQUIRE(gain_n == 1 || gain_n == H, "norm_add: %d gains for %d channels", gain_n, H);
+  NINFER_REQUIRE(dtype == kF32 || dtype == kBF16, "norm_add: unknown dtype %d", dtype);
+  const int block = H >= 1024 ? 1024 : (H + 63) / 64 * 64;
+  if (dtype == kF32)
+    norm_add_kernel<float><<<T, block, 0, stream>>>(x, (const float*)y, gain, gain_n, H, eps);
+  else
+    norm_add_kernel<bf16><<<T, block, 0, stream>>>(x, (const bf16*)y, gain, gain_n, H, eps);
+  NINFER_LAUNCH_CHECK();
+  return 0;
+}
+
+extern "C" int ninfer_gated_rmsnorm(const float* o, const void* gate, int gate_stride,
+                                    const float* w, void* out, int T, int N, float eps, int dtype,
+                                    hipStream_t stream) {
+  NINFER_REQUIRE(T > 0 && N > 0 && gate_stride >= N, "gated_rmsnorm: T=%d N=%d gate stride %d", T,
+                 N, gate_stride);
+  NINFER_REQUIRE(dtype == kF32 || dtype == kBF16, "gated_rmsnorm: unknown dtype %d", dtype);
+  const int block = N >= 1024 ? 1024 : (N + 63) / 64 * 64;
+  if (dtype == kF32)
+    gated_rmsnorm_kernel<float><<<T, block, 0, stream>>>(o, (const float*)gate, gate_stride, w,
+                                                         (float*)out, N, eps);
+  else
+    gated_rmsnorm_kernel<bf16><<<T, block, 0, stream>>>(o, (const bf16*)gate, gate_stride, w,
+                                                        (bf16*)out, N, eps);
+  NINFER_LAUNCH_CHECK();
+  return 0;
+}

@@ -67,7 +67,7 @@ class ModelRunner:
         for call in spec.plan:
             mixer = spec.blocks[call.layer].mixer
             needs.append(mixer.cache_need() if call.cache_from is None else None)
-            n = mixer.state_floats()
+            n = spec.blocks[call.layer].state_floats()
             self._state_range.append(slice(floats, floats + n) if n else None)
             floats += n
         own = {"float32": 4, "bfloat16": 2}

@@ -88,6 +88,19 @@ class _QkvRopeArgs(ctypes.Structure):
                 ("write_kv", ctypes.c_int)]
 
 
+class _LatentArgs(ctypes.Structure):
+    _fields_ = [("dkv", ctypes.c_void_p), ("q", ctypes.c_void_p), ("q_abs", ctypes.c_void_p),
+                ("pool", ctypes.c_void_p), ("out", ctypes.c_void_p), ("gate", ctypes.c_void_p),
+                ("norm_w", ctypes.c_void_p), ("freq", ctypes.c_void_p),
+                ("block_table", ctypes.c_void_p), ("positions", ctypes.c_void_p),
+                ("row_seq", ctypes.c_void_p), ("dkv_stride", ctypes.c_int),
+                ("gate_stride", ctypes.c_int), ("bt_stride", ctypes.c_int), ("T", ctypes.c_int),
+                ("Hq", ctypes.c_int), ("dim", ctypes.c_int), ("R", ctypes.c_int),
+                ("rd", ctypes.c_int), ("rot_n", ctypes.c_int), ("page_size", ctypes.c_int),
+                ("window", ctypes.c_int), ("write_kv", ctypes.c_int), ("dtype", ctypes.c_int),
+                ("eps", ctypes.c_float), ("magnitude", ctypes.c_float), ("scale", ctypes.c_float)]
+
+
 def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
     return None if t is None else t.data_ptr()
 
@@ -843,6 +856,180 @@ class HipOps:
                     "chunks": n_chunks.value}
         self._ok(self.lib.ninfer_paged_attention(ctypes.byref(args),
                                                  1 if self.force_generic else 0, self._stream()))
+
+    # ---- sublayers with the norm on their output -----------------------------------
+    def short_conv(self, x, w, state, ctx, out):
+        """out = x + conv(x): per channel, conv(x)_t = sum_j w[:, j] x_(t - taps + 1 + j) over
+        the rows of each request; the taps - 1 inputs before a step's first row come from
+        `state` ([slots, >= (taps - 1) * H] 32-bit, a view whose rows may lie apart), which is
+        moved on to the step's last inputs. x: the 32-bit rows [T, H]; w: [H, taps] 32-bit."""
+        _dev(x, "x", torch.float32, 2)
+        _dev(w, "w", torch.float32, 2)
+        _dev(out, "out", dims=2)
+        t, h = x.shape
+        taps = w.shape[1]
+        _need(w.shape[0] == h and out.shape == (t, h), "short_conv: shapes")
+        _need(out.dtype in _DT, f"short_conv: out of {out.dtype}")
+        _need(state.is_cuda and state.dtype == torch.float32 and state.dim() == 2
+              and state.stride(1) == 1 and state.shape[1] >= (taps - 1) * h,
+              "short_conv: the state must be 32-bit rows of at least (taps - 1) * H numbers")
+        _need(ctx.T == t, "short_conv: rows differ from the step's")
+        self._ok(self.lib.ninfer_short_conv(
+            ctypes.c_void_p(x.data_ptr()), ctypes.c_void_p(w.data_ptr()),
+            ctypes.c_void_p(state.data_ptr()), ctypes.c_longlong(state.stride(0)),
+            ctypes.c_void_p(out.data_ptr()), ctypes.c_void_p(ctx.row_seq.data_ptr()),
+            ctypes.c_void_p(ctx.seq_row_start.data_ptr()), ctypes.c_void_p(ctx.seq_slots.data_ptr()),
+            t, ctx.S, h, taps, 1 if ctx.max_qlen == 1 else 0, _DT[out.dtype], self._stream()))
+
+    def norm_add(self, residual, y, gain, eps):
+        """residual += y rsqrt(mean(y^2) + eps) gain; gain holds one number or one per column."""
+        _dev(residual, "residual", torch.float32, 2)
+        _dev(y, "y", dims=2)
+        _dev(gain, "gain", torch.float32, 1)
+        _need(y.shape == residual.shape and y.dtype in _DT, "norm_add: y does not fit the residual")
+        _need(gain.shape[0] in (1, y.shape[1]), "norm_add: one gain, or one per column")
+        self._ok(self.lib.ninfer_norm_add(
+            ctypes.c_void_p(residual.data_ptr()), ctypes.c_void_p(y.data_ptr()),
+            ctypes.c_void_p(gain.data_ptr()), gain.shape[0], y.shape[0], y.shape[1],
+            ctypes.c_float(eps), _DT[y.dtype], self._stream()))
+
+    def gated_rmsnorm(self, o, gate, weight, eps, out):
+        """out = o rsqrt(mean(o^2) + eps) weight sigmoid(gate), the mean over the whole row.
+        o: [T, N] 32-bit; gate: [T, N] columns of a wider row-major tensor (a view)."""
+        _dev(o, "o", torch.float32, 2)
+        _dev(weight, "weight", torch.float32, 1)
+        _dev(out, "out", dims=2)
+        t, n = o.shape
+        _need(out.shape == (t, n) and weight.shape[0] == n and out.dtype in _DT,
+              "gated_rmsnorm: shapes")
+        _need(gate.is_cuda and gate.dtype == out.dtype and gate.shape == (t, n)
+              and gate.stride(1) == 1, "gated_rmsnorm: the gate must be [T, N] columns of rows")
+        self._ok(self.lib.ninfer_gated_rmsnorm(
+            ctypes.c_void_p(o.data_ptr()), ctypes.c_void_p(gate.data_ptr()),
+            gate.stride(0) if t > 1 else max(n, gate.stride(0)),
+            ctypes.c_void_p(weight.data_ptr()), ctypes.c_void_p(out.data_ptr()), t, n,
+            ctypes.c_float(eps), _DT[out.dtype], self._stream()))
+
+    def lightning_attention(self, qkv, q_off, k_off, v_off, heads, dim, vdim, decay, state, ctx,
+                            out):
+        """Linear attention with a decay per head over the rows of each request:
+        S <- decay_h S + k v^T, out = S^T q with q, k, v = silu of the columns of `qkv` at
+        q_off, k_off (heads x dim) and v_off (heads x vdim). `state` ([slots, >= heads * dim *
+        vdim] 32-bit view) holds every request's S between steps. out: [T, heads * vdim] 32-bit."""
+        _dev(qkv, "qkv", dims=2)
+        _dev(decay, "decay", torch.float32, 1)
+        _dev(out, "out", torch.float32, 2)
+        t = qkv.shape[0]
+        _need(qkv.dtype in _DT, f"lightning_attention: rows of {qkv.dtype}")
+        _need(decay.shape[0] == heads and out.shape == (t, heads * vdim) and ctx.T == t,
+              "lightning_attention: shapes")
+        for off, n in ((q_off, heads * dim), (k_off, heads * dim), (v_off, heads * vdim)):
+            _need(0 <= off and off + n <= qkv.shape[1], "lightning_attention: columns outside the rows")
+        _need(state.is_cuda and state.dtype == torch.float32 and state.dim() == 2
+              and state.stride(1) == 1 and state.shape[1] >= heads * dim * vdim,
+              "lightning_attention: the state must be 32-bit rows of heads * dim * vdim numbers")
+        self._ok(self.lib.ninfer_lightning_attention(
+            ctypes.c_void_p(qkv.data_ptr()), qkv.shape[1], q_off, k_off, v_off,
+            ctypes.c_void_p(decay.data_ptr()), ctypes.c_void_p(state.data_ptr()),
+            ctypes.c_longlong(state.stride(0)), ctypes.c_void_p(out.data_ptr()),
+            ctypes.c_void_p(ctx.seq_row_start.data_ptr()), ctypes.c_void_p(ctx.seq_slots.data_ptr()),
+            t, ctx.S, heads, dim, vdim, _DT[qkv.dtype], self._stream()))
+
+    def _latent_args(self, ctx, pool, block_table, heads, dim, rank, rot_dim, rot_n, page_size,
+                     dtype):
+        _dev(pool, "pool", dtype, 3)
+        _need(pool.shape[1:] == (page_size, rank + rot_dim),
+              f"latent attention: pool {tuple(pool.shape)} does not fit pages of {page_size} rows "
+              f"of {rank + rot_dim}")
+        _dev(block_table, "block_table", torch.int32, 2)
+        _need(block_table.shape[0] == ctx.S, "latent attention: block table rows != requests")
+        a = _LatentArgs()
+        a.pool, a.block_table = pool.data_ptr(), block_table.data_ptr()
+        a.positions, a.row_seq = ctx.positions.data_ptr(), ctx.row_seq.data_ptr()
+        a.bt_stride, a.T, a.Hq, a.dim, a.R, a.rd, a.rot_n = \
+            block_table.shape[1], ctx.T, heads, dim, rank, rot_dim, rot_n
+        a.page_size, a.dtype = page_size, _DT[dtype]
+        return a
+
+    def latent_kv_write(self, dkv, q, q_abs, pool, block_table, ctx, heads, dim, rank, rot_dim,
+                        norm_w, eps, freq, rot_n, magnitude, page_size, write_kv=True):
+        """Per row: the first `rank` columns of `dkv` normed (x rsqrt(mean(x^2) + eps) norm_w)
+        and the next `rot_dim`, turned by the row's position, go to the request's page of
+        `pool` [pages, page_size, rank + rot_dim]; the rotated part of every head of `q`
+        ([T, heads * (dim + rot_dim)]) is turned and written behind the first `rank` numbers of
+        the head's row of `q_abs` [T, heads, rank + rot_dim] (32-bit). Pair (i, i + rot_n / 2)
+        of the first rot_n rotated numbers turns by pos * freq[i]; cos and sin times `magnitude`."""
+        _need(dkv.is_cuda and dkv.dim() == 2 and dkv.stride(1) == 1 and dkv.shape[1] >= rank + rot_dim,
+              "latent_kv_write: dkv must be rows of at least rank + rot_dim columns")
+        _dev(q, "q", dkv.dtype, 2)
+        _dev(q_abs, "q_abs", torch.float32, 3)
+        _dev(norm_w, "norm_w", torch.float32, 1)
+        t = ctx.T
+        _need(dkv.shape[0] == t and q.shape == (t, heads * (dim + rot_dim))
+              and q_abs.shape == (t, heads, rank + rot_dim) and norm_w.shape[0] == rank,
+              "latent_kv_write: shapes")
+        a = self._latent_args(ctx, pool, block_table, heads, dim, rank, rot_dim, rot_n, page_size,
+                              dkv.dtype)
+        if rot_n:
+            _dev(freq, "freq", torch.float32, 1)
+            _need(freq.shape[0] == rot_n // 2, "latent_kv_write: table size != rot_n / 2")
+            a.freq = freq.data_ptr()
+        a.dkv, a.q, a.q_abs, a.norm_w = dkv.data_ptr(), q.data_ptr(), q_abs.data_ptr(), norm_w.data_ptr()
+        a.dkv_stride = dkv.stride(0) if t > 1 else max(dkv.shape[1], dkv.stride(0))
+        a.eps, a.magnitude, a.scale, a.write_kv = eps, magnitude, 1.0, 1 if write_kv else 0
+        self._ok(self.lib.ninfer_latent_kv_write(ctypes.byref(a), self._stream()))
+
+    def latent_attention(self, q_abs, pool, block_table, ctx, heads, rank, rot_dim, page_size,
+                         scale, out, gate=None, window=None):
+        """Softmax attention of q_abs [T, heads, rank + rot_dim] (32-bit) over the rows of the
+        requests' pages of `pool` (every head reads the same rows): scores (q . row) * scale
+        over positions <= the row's own (within `window` if given), out[t, h] = sum_j p_j
+        row_j[:rank], times sigmoid(gate[t, h]) when `gate` ([T, heads] columns of a wider
+        tensor, a view) is given. out: [T, heads * rank]."""
+        _dev(q_abs, "q_abs", torch.float32, 3)
+        _dev(out, "out", pool.dtype, 2)
+        t = ctx.T
+        _need(q_abs.shape == (t, heads, rank + rot_dim) and out.shape == (t, heads * rank),
+              "latent_attention: shapes")
+        a = self._latent_args(ctx, pool, block_table, heads, 0, rank, rot_dim, 0, page_size,
+                              pool.dtype)
+        a.q_abs, a.out, a.scale, a.window = q_abs.data_ptr(), out.data_ptr(), scale, int(window or 0)
+        if gate is not None:
+            _need(gate.is_cuda and gate.dtype == pool.dtype and gate.shape == (t, heads)
+                  and gate.stride(1) == 1, "latent_attention: the gate must be [T, heads] columns")
+            a.gate = gate.data_ptr()
+            a.gate_stride = gate.stride(0) if t > 1 else max(heads, gate.stride(0))
+        self._ok(self.lib.ninfer_latent_attention(ctypes.byref(a), self._stream()))
+
+    def head_index(self, ctx, heads):
+        """(offsets [heads + 1], index [T * heads]) for products that every head runs with
+        weights of its own on its own columns of the rows: with the rows viewed as [T * heads,
+        columns of a head], group h owns the sorted rows h * T .. (h + 1) * T - 1, and sorted
+        row h * T + t is row t * heads + h. Made once per step and kept in its scratch."""
+        key = ("head_index", heads)
+        if key not in ctx.scratch:
+            t = ctx.T
+            offsets = torch.arange(0, (heads + 1) * t, t, dtype=torch.int32, device=ctx.device)
+            index = (torch.arange(t, dtype=torch.int32, device=ctx.device)[None, :] * heads
+                     + torch.arange(heads, dtype=torch.int32, device=ctx.device)[:, None]).reshape(-1)
+            ctx.scratch[key] = (offsets, index.contiguous())
+        return ctx.scratch[key]
+
+    def per_head_linear(self, x, w, out, ctx, k, n):
+        """out[t, h, :n] = x[t, h, :k] w[h]^T for every head: x [T, heads, >= k], w [heads, n, k],
+        out [T, heads, >= n] (32-bit or x's dtype); columns beyond k and n are left alone. Runs
+        as one grouped product (the groups are the heads)."""
+        _dev(x, "x", dims=3)
+        _dev(w, "w", x.dtype, 3)
+        _dev(out, "out", dims=3)
+        t, heads = x.shape[0], x.shape[1]
+        _need(w.shape == (heads, n, k) and x.shape[2] >= k and out.shape[:2] == (t, heads)
+              and out.shape[2] >= n, "per_head_linear: shapes")
+        _need(out.dtype in (x.dtype, torch.float32), "per_head_linear: bad out dtype")
+        offsets, index = self.head_index(ctx, heads)
+        self._gemm(x.view(t * heads, x.shape[2]), w, out.view(t * heads, out.shape[2]),
+                   m=t * heads, n=n, k=k, offsets=offsets, a_index=index, c_index=index,
+                   groups=heads, w_group_stride=n * k)
 
     # ---- sampling -------------------------------------------------------------------
     FEW_TOKENS = 64   # most tokens a row may keep (top_k) for the two-launch sampling path

@@ -1,4 +1,5 @@
+from . import getodra  # registers Getodra
 from . import qwen2_moe  # registers Qwen2MoeForCausalLM
 from .spec import LayerCall, ModelSpec
 
-__all__ = ["LayerCall", "ModelSpec", "qwen2_moe"]
+__all__ = ["LayerCall", "ModelSpec", "getodra", "qwen2_moe"]

@@ -76,7 +76,8 @@ class CacheView:
 class CallInfo:
     """How one entry of the layer plan runs: which cache it uses, whether it
     writes it (false when it reads another call's cache), and the slice of the
-    per-request state that belongs to its mixer ([slots, floats], or None)."""
+    per-request state that belongs to it ([slots, floats], or None): a block's for the block,
+    the mixer's for the mixer."""
     cache: Optional[CacheView] = None
     writes_cache: bool = True
     state: Optional[torch.Tensor] = None
@@ -287,6 +288,12 @@ class Block(Part):
     """Arrangement of norms, mixer and feed-forward around the residual."""
 
     mixer: Mixer
+
+    def state_floats(self) -> int:
+        """32-bit numbers of per-request state of one run of this block: the mixer's, and
+        whatever the block's other parts keep (a block that has such parts adds them and hands
+        each its columns of `CallInfo.state`)."""
+        return self.mixer.state_floats()
 
     def forward(self, ctx: StepContext, residual: torch.Tensor,
                 pending: Optional[torch.Tensor], call: CallInfo) -> Optional[torch.Tensor]:

@@ -11,7 +11,7 @@ from __future__ import annotations
 from typing import List, Optional
 
 from ..registry import register_part
-from .base import Block, CallInfo, FeedForward, Mixer, Norm, Part, StepContext
+from .base import Block, CallInfo, FeedForward, Mixer, Norm, Part, StepContext, settle
 
 
 class PreNormBlock(Block):
@@ -32,3 +32,63 @@ class PreNormBlock(Block):
 
 
 register_part("block", "pre_norm", PreNormBlock)
+
+
+class OutputNormBlock(Block):
+    """A block whose norms sit on the sublayers' outputs: x += norm1(mixer(in1(x))), then
+    x += norm2(feed_forward(in2(x))). The sublayers read the 32-bit residual itself, through an
+    optional input part each (`mixer_input`, `ff_input`: e.g. a short convolution with state of
+    its own); `feed_forward` may be None (a layer with a mixer only). The block adds into the
+    residual itself and hands nothing on. Its per-request state holds, in this order, the
+    mixer input's, the mixer's and the feed-forward input's."""
+
+    def __init__(self, mixer: Mixer, mixer_norm: Part, feed_forward: Optional[FeedForward] = None,
+                 ff_norm: Optional[Part] = None, mixer_input: Optional[Part] = None,
+                 ff_input: Optional[Part] = None):
+        if (feed_forward is None) != (ff_norm is None):
+            raise ValueError("a feed-forward and its norm come together or not at all")
+        self.mixer = mixer
+        self.mixer_norm = mixer_norm
+        self.feed_forward = feed_forward
+        self.ff_norm = ff_norm
+        self.mixer_input = mixer_input
+        self.ff_input = ff_input if feed_forward is not None else None
+
+    def children(self) -> List[Part]:
+        return [p for p in (self.mixer_input, self.mixer, self.mixer_norm, self.ff_input,
+                            self.feed_forward, self.ff_norm) if p is not None]
+
+    def _state_parts(self):
+        a = self.mixer_input.state_floats() if self.mixer_input is not None else 0
+        b = self.mixer.state_floats()
+        c = self.ff_input.state_floats() if self.ff_input is not None else 0
+        return a, b, c
+
+    def state_floats(self) -> int:
+        return sum(self._state_parts())
+
+    def _read(self, ctx: StepContext, residual, part, state):
+        if part is not None:
+            return part.forward(ctx, residual, state)
+        if residual.dtype == ctx.act_dtype:
+            return residual
+        return residual.to(ctx.act_dtype)
+
+    def forward(self, ctx: StepContext, residual, pending, call: CallInfo):
+        settled = settle(ctx, residual, pending)
+        if settled is not None:
+            residual.add_(settled)
+        a, b, c = self._state_parts()
+        st = call.state
+        h = self._read(ctx, residual, self.mixer_input, st[:, :a] if a else None)
+        inner = CallInfo(cache=call.cache, writes_cache=call.writes_cache,
+                         state=st[:, a:a + b] if b else None)
+        self.mixer_norm.add(ctx, residual, self.mixer.forward(ctx, h, residual, inner))
+        if self.feed_forward is not None:
+            h = self._read(ctx, residual, self.ff_input, st[:, a + b:a + b + c] if c else None)
+            y = settle(ctx, residual, self.feed_forward.forward(ctx, h, residual))
+            self.ff_norm.add(ctx, residual, y)
+        return None
+
+
+register_part("block", "output_norm", OutputNormBlock)

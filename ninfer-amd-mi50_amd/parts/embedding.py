@@ -20,8 +20,11 @@ from .base import Part, StepContext, WeightBinder
 
 class TokenEmbedding(Part):
     def __init__(self, prefix: str, vocab: int, hidden: int, positions: int = 0,
-                 position_prefix: Optional[str] = None):
+                 position_prefix: Optional[str] = None, leaf: str = "weight"):
+        """`leaf`: what follows the prefixes in the tensors' names ('' when a prefix is the
+        whole name)."""
         self.prefix = prefix
+        self.leaf = leaf
         self.vocab = vocab
         self.hidden = hidden
         self.positions = positions   # rows of the table of learned positions (0: none)
@@ -32,15 +35,15 @@ class TokenEmbedding(Part):
         self.position_table: Optional[torch.Tensor] = None
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
-        specs = {self.prefix + "weight": TensorSpec((self.vocab, self.hidden))}
+        specs = {self.prefix + self.leaf: TensorSpec((self.vocab, self.hidden))}
         if self.positions:
-            specs[self.position_prefix + "weight"] = TensorSpec((self.positions, self.hidden))
+            specs[self.position_prefix + self.leaf] = TensorSpec((self.positions, self.hidden))
         return specs
 
     def bind(self, w: WeightBinder) -> None:
-        self.table = w.matrix(self.prefix + "weight")
+        self.table = w.matrix(self.prefix + self.leaf)
         if self.positions:
-            self.position_table = w.matrix(self.position_prefix + "weight")
+            self.position_table = w.matrix(self.position_prefix + self.leaf)
 
     def max_positions(self) -> Optional[int]:
         return self.positions or None
@@ -54,8 +57,9 @@ class TokenEmbedding(Part):
 
 class LMHead(Part):
     def __init__(self, prefix: str, vocab: int, hidden: int,
-                 tied_to: Optional[TokenEmbedding] = None):
+                 tied_to: Optional[TokenEmbedding] = None, leaf: str = "weight"):
         self.prefix = prefix
+        self.leaf = leaf
         self.vocab = vocab
         self.hidden = hidden
         self.tied_to = tied_to
@@ -64,17 +68,17 @@ class LMHead(Part):
     def tensor_specs(self) -> Dict[str, TensorSpec]:
         if self.tied_to is not None:
             return {}
-        return {self.prefix + "weight": TensorSpec((self.vocab, self.hidden))}
+        return {self.prefix + self.leaf: TensorSpec((self.vocab, self.hidden))}
 
     def unused_tensor_specs(self) -> Dict[str, TensorSpec]:
         # a checkpoint of a tied model may still carry the head: a copy of the table
         if self.tied_to is not None:
-            return {self.prefix + "weight": TensorSpec((self.vocab, self.hidden))}
+            return {self.prefix + self.leaf: TensorSpec((self.vocab, self.hidden))}
         return {}
 
     def bind(self, w: WeightBinder) -> None:
         if self.tied_to is None:
-            self.weight = w.matrix(self.prefix + "weight")
+            self.weight = w.matrix(self.prefix + self.leaf)
 
     def forward(self, ctx: StepContext, normed_rows: torch.Tensor) -> torch.Tensor:
         weight = self.tied_to.table if self.tied_to is not None else self.weight

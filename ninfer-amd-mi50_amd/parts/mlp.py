@@ -18,8 +18,12 @@ from .base import FeedForward, StepContext, WeightBinder
 
 
 class SwiGLU(FeedForward):
-    def __init__(self, prefix: str, hidden: int, inner: int, act: str = "silu", bias: bool = False):
+    def __init__(self, prefix: str, hidden: int, inner: int, act: str = "silu", bias: bool = False,
+                 names=("gate_proj.weight", "up_proj.weight", "down_proj.weight")):
+        """`names`: what follows the prefix in the names of the gate's, the other half's and the
+        down product's weights."""
         self.prefix = prefix
+        self.names = tuple(names)
         self.hidden = hidden
         self.inner = inner
         self.act = act   # the gate's activation, by config.json's name: 'silu' | 'gelu_pytorch_tanh'
@@ -31,9 +35,9 @@ class SwiGLU(FeedForward):
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
         p = self.prefix
-        specs = {p + "gate_proj.weight": TensorSpec((self.inner, self.hidden)),
-                 p + "up_proj.weight": TensorSpec((self.inner, self.hidden)),
-                 p + "down_proj.weight": TensorSpec((self.hidden, self.inner))}
+        specs = {p + self.names[0]: TensorSpec((self.inner, self.hidden)),
+                 p + self.names[1]: TensorSpec((self.inner, self.hidden)),
+                 p + self.names[2]: TensorSpec((self.hidden, self.inner))}
         if self.bias:
             specs[p + "gate_proj.bias"] = TensorSpec((self.inner,), "bias")
             specs[p + "up_proj.bias"] = TensorSpec((self.inner,), "bias")
@@ -44,9 +48,9 @@ class SwiGLU(FeedForward):
         p = self.prefix
         self.w_gate_up = torch.empty((2 * self.inner, self.hidden), dtype=w.act_dtype,
                                      device=w.device)
-        w.matrix_into(p + "gate_proj.weight", self.w_gate_up[:self.inner])
-        w.matrix_into(p + "up_proj.weight", self.w_gate_up[self.inner:])
-        self.w_down = w.matrix(p + "down_proj.weight")
+        w.matrix_into(p + self.names[0], self.w_gate_up[:self.inner])
+        w.matrix_into(p + self.names[1], self.w_gate_up[self.inner:])
+        self.w_down = w.matrix(p + self.names[2])
         if self.bias:
             self.b_gate_up = torch.cat([w.float32(p + "gate_proj.bias"), w.float32(p + "up_proj.bias")])
             w.hold(p + "gate_proj.bias", self.b_gate_up[:self.inner])

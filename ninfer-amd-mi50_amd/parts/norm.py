@@ -12,21 +12,28 @@ import torch
 
 from ..registry import register_part
 from ..weights.source import TensorSpec
-from .base import Norm, PendingRows, StepContext, WeightBinder
+from .base import Norm, Part, PendingRows, StepContext, WeightBinder
 
 
 class RMSNorm(Norm):
-    def __init__(self, prefix: str, size: int, eps: float):
+    def __init__(self, prefix: str, size: int, eps: float, leaf: str = "weight",
+                 single_gain: bool = False):
+        """`leaf`: what follows the prefix in the gain's name ('' when the prefix is the whole
+        name). `single_gain`: the checkpoint holds one number (shape []) for all columns."""
         self.prefix = prefix
         self.size = size
         self.eps = eps
+        self.leaf = leaf
+        self.single_gain = single_gain
         self.gain: Optional[torch.Tensor] = None
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
-        return {self.prefix + "weight": TensorSpec((self.size,), "gain")}
+        return {self.prefix + self.leaf: TensorSpec(() if self.single_gain else (self.size,), "gain")}
 
     def bind(self, w: WeightBinder) -> None:
-        self.gain = w.float32(self.prefix + "weight")
+        self.gain = w.float32(self.prefix + self.leaf)
+        if self.single_gain:   # the kernel reads one gain per column
+            self.gain = self.gain.reshape(1).expand(self.size).contiguous()
 
     def forward(self, ctx: StepContext, residual, pending):
         out = ctx.empty((residual.shape[0], self.size))
@@ -45,4 +52,27 @@ class RMSNorm(Norm):
         return out
 
 
+class OutputRMSNorm(Part):
+    """The norm of a block that norms what a sublayer gives back, not what it reads:
+    residual += y rsqrt(mean(y^2) + eps) gain, in 32-bit, where the gain is one number for
+    all columns (`single_gain`, shape []) or one per column."""
+
+    def __init__(self, tensor: str, size: int, eps: float, single_gain: bool = True):
+        self.tensor = tensor
+        self.size = size
+        self.eps = eps
+        self.single_gain = single_gain
+        self.gain: Optional[torch.Tensor] = None
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        return {self.tensor: TensorSpec(() if self.single_gain else (self.size,), "gain")}
+
+    def bind(self, w: WeightBinder) -> None:
+        self.gain = w.float32(self.tensor).reshape(-1)
+
+    def add(self, ctx: StepContext, residual: torch.Tensor, y: torch.Tensor) -> None:
+        ctx.ops.norm_add(residual, y, self.gain, self.eps)
+
+
 register_part("norm", "rmsnorm", RMSNorm)
+register_part("norm", "output_rmsnorm", OutputRMSNorm)

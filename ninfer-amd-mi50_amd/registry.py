@@ -13,7 +13,7 @@ from typing import Any, Callable, Dict, Tuple
 
 _ARCHITECTURES: Dict[str, Tuple[Callable[[dict], Any], Callable[[Any], Any]]] = {}
 _PARTS: Dict[str, Dict[str, Callable[..., Any]]] = {
-    "mixer": {}, "feed_forward": {}, "norm": {}, "position": {}, "block": {},
+    "mixer": {}, "feed_forward": {}, "norm": {}, "position": {}, "block": {}, "input": {},
 }
 
 
@@ -36,7 +36,7 @@ def resolve_architecture(name: str) -> Tuple[Callable[[dict], Any], Callable[[An
 
 def register_part(kind: str, name: str, factory: Callable[..., Any]) -> None:
     """Register a part factory under kind 'mixer', 'feed_forward', 'norm',
-    'position' or 'block'."""
+    'position', 'block' or 'input' (what a sublayer's input passes through first)."""
     if kind not in _PARTS:
         raise KeyError(f"unknown part kind {kind!r}; kinds: {', '.join(sorted(_PARTS))}")
     _PARTS[kind][name] = factory
