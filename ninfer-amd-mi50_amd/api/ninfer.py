@@ -72,12 +72,20 @@ class Session:
 
 
 class Ninfer:
-    def __init__(self, model_dir: Optional[str] = None, max_context: int = 32768,
+    def __init__(self, model_dir: Optional[str] = None, max_context: Optional[int] = 32768,
                  prefill_chunk: int = 512, num_sequences: int = 1, dtype: str = "bfloat16",
                  page_size: int = 16, num_pages: Optional[int] = None, use_graph: bool = False,
                  random_config: Optional[dict] = None, random_seed: int = 0,
                  random_weights_dtype: Optional[str] = None, kv_bytes: Optional[int] = None,
                  check_pages: bool = False):
+        if max_context is None:
+            # as many positions as the model's parts allow (a table of learned positions has
+            # so many rows), and no more than the reference's default
+            from ..config.base import read_config_json
+            from ..loading import build_spec
+            raw = random_config if model_dir is None else read_config_json(model_dir)
+            limit = build_spec(raw)[1].max_positions() if raw is not None else None
+            max_context = 32768 if limit is None else min(32768, limit)
         self.options = EngineOptions(dtype=dtype, max_context=max_context,
                                      prefill_chunk=prefill_chunk, num_sequences=num_sequences,
                                      page_size=page_size, num_pages=num_pages,

@@ -28,7 +28,9 @@ def build_parser() -> argparse.ArgumentParser:
                     help="a prompt as comma-separated token ids (may be given several times)")
     ap.add_argument("--prompt-file", help="JSON file: a list of lists of token ids")
     ap.add_argument("--random-prompts", help="comma-separated lengths of seeded random prompts")
-    ap.add_argument("--max-context", type=int, default=32768, help="KV capacity in tokens per request")
+    ap.add_argument("--max-context", type=int, default=None,
+                    help="KV capacity in tokens per request (default: 32768, or the model's most "
+                         "positions where its parts bound them)")
     ap.add_argument("--prefill-chunk", type=int, default=512, help="token budget of one step")
     ap.add_argument("--max-new", type=int, default=512, help="new tokens per generation")
     ap.add_argument("--temperature", type=float, default=0.7, help="sampling temperature (0 = greedy)")
@@ -88,7 +90,7 @@ def main(argv: Optional[List[str]] = None) -> int:
             rng = random.Random(args.seed or 1234)
             for n in args.random_prompts.split(","):
                 prompts.append([rng.randrange(eng.vocab) for _ in range(int(n))])
-        log(f"engine ready in {time.time() - t0:.1f} s: vocab={eng.vocab} ctx={args.max_context} "
+        log(f"engine ready in {time.time() - t0:.1f} s: vocab={eng.vocab} ctx={eng.max_context} "
             f"chunk={args.prefill_chunk} seqs={args.max_seqs} dtype={dtype}")
         stop = [args.eos_id] if args.eos_id is not None else None
         if not prompts:

@@ -870,13 +870,18 @@ class HipOps:
         taps = w.shape[1]
         _need(w.shape[0] == h and out.shape == (t, h), "short_conv: shapes")
         _need(out.dtype in _DT, f"short_conv: out of {out.dtype}")
-        _need(state.is_cuda and state.dtype == torch.float32 and state.dim() == 2
-              and state.stride(1) == 1 and state.shape[1] >= (taps - 1) * h,
-              "short_conv: the state must be 32-bit rows of at least (taps - 1) * H numbers")
+        if taps == 1 and state is None:   # one tap keeps nothing
+            state_ptr, state_stride = None, 0
+        else:
+            _need(state is not None and state.is_cuda and state.dtype == torch.float32
+                  and state.dim() == 2 and state.stride(1) == 1
+                  and state.shape[1] >= (taps - 1) * h,
+                  "short_conv: the state must be 32-bit rows of at least (taps - 1) * H numbers")
+            state_ptr, state_stride = state.data_ptr(), state.stride(0)
         _need(ctx.T == t, "short_conv: rows differ from the step's")
         self._ok(self.lib.ninfer_short_conv(
             ctypes.c_void_p(x.data_ptr()), ctypes.c_void_p(w.data_ptr()),
-            ctypes.c_void_p(state.data_ptr()), ctypes.c_longlong(state.stride(0)),
+            ctypes.c_void_p(state_ptr), ctypes.c_longlong(state_stride),
             ctypes.c_void_p(out.data_ptr()), ctypes.c_void_p(ctx.row_seq.data_ptr()),
             ctypes.c_void_p(ctx.seq_row_start.data_ptr()), ctypes.c_void_p(ctx.seq_slots.data_ptr()),
             t, ctx.S, h, taps, 1 if ctx.max_qlen == 1 else 0, _DT[out.dtype], self._stream()))

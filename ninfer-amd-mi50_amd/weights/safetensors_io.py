@@ -131,7 +131,7 @@ def write_safetensors(path: str, tensors: Iterable[Tuple[str, torch.Tensor]]) ->
             t = t.detach().to("cpu").contiguous()
             if t.dtype not in _TAG_OF:
                 raise WeightError(f"cannot write tensor '{name}' of dtype {t.dtype}")
-            raw = t.view(torch.uint8).numpy().tobytes() if t.numel() else b""
+            raw = t.reshape(-1).view(torch.uint8).numpy().tobytes() if t.numel() else b""   # (reshape: a single number has no dimension to view through)
             items.append((name, {"dtype": _TAG_OF[t.dtype], "shape": list(t.shape),
                                  "data_offsets": [offset, offset + len(raw)]}))
             data.write(raw)

@@ -199,7 +199,7 @@ def run_schedule(runner, steps: List[Step]) -> Dict[str, torch.Tensor]:
                 o += len(want)
         for rid in end:
             runner.close(slots.pop(rid))
-    return {rid: torch.cat(v) for rid, v in rows.items()}
+    return {rid: torch.cat(v) for rid, v in rows.items() if v}   # (a schedule may want no row of a request)
 
 
 class DictSource:
