@@ -16,6 +16,13 @@ step's fraction of that); decode at batch 1 and 64 under "points"; and under
 those batches (untimed; 0.0 when the replays are exact).
 Peaks: HBM 8 TB/s; dense bf16 MFMA 2.5 PFLOP/s (fp32 157.3 TFLOP/s).
 
+    python bench.py --scenario designs [--sizes small,medium]
+
+is a third measurement, again with a JSON line of its own: Getodra (latent attention and
+lightning attention layers with input convolutions and output norms) beside a dense
+Qwen2-style model of the same width, depth, heads and feed-forward size, both with random
+weights: prompt portions of 512 and 2,048 tokens and decode steps at batch 1, 8 and 64.
+
     python bench.py --scenario long [--model 57b-a14b] [--requests 8] [--prompt 32768] [--new 256]
 
 is another measurement with a JSON line of its own: the scheduler serves
@@ -75,7 +82,9 @@ def main() -> int:
                          "prefill with device events, with the bytes and flops of each kind, its "
                          "floor and the fraction of it reached (untimed runs of their own; the "
                          "table goes to stderr and under \"profile\")")
-    ap.add_argument("--scenario", default="decode", choices=["decode", "long"])
+    ap.add_argument("--scenario", default="decode", choices=["decode", "long", "designs"])
+    ap.add_argument("--sizes", default="small,medium",
+                    help="--scenario designs: which of the layer sizes to run (small, medium)")
     ap.add_argument("--requests", type=int, default=8, help="--scenario long: concurrent requests")
     ap.add_argument("--prompt", type=int, default=32768, help="--scenario long: prompt tokens")
     ap.add_argument("--new", type=int, default=256, help="--scenario long: new tokens a request")
@@ -107,6 +116,8 @@ def main() -> int:
     page = 16
     if args.scenario == "long":
         return long_scenario(args, raw, model_name, layers_full)
+    if args.scenario == "designs":
+        return designs_scenario(args)
     max_b = args.batch if args.no_points else max(args.batch, 64)
     ctx = args.context
     opt = EngineOptions(dtype=args.dtype, max_context=ctx, prefill_chunk=max(args.prefill_tokens, max_b),
@@ -451,6 +462,112 @@ def main() -> int:
             print(f"[bench] WARNING: replayed steps differ from eager steps by {worst}",
                   file=sys.stderr, flush=True)
     print(json.dumps(result), flush=True)
+    return 0
+
+
+DESIGN_SIZES = {
+    # width, feed-forward, layers, heads, head size (attention: unrotated + rotated = head), latent
+    "small": dict(width=1024, ff=2816, layers=8, heads=8, head=128, rot=32, vdim=64, rank=256,
+                  vocab=32000, positions=4096),
+    "medium": dict(width=2048, ff=5632, layers=8, heads=16, head=128, rot=64, vdim=128, rank=512,
+                   vocab=32000, positions=4096),
+}
+
+
+def getodra_config(z: dict) -> dict:
+    """Three latent-attention layers to one lightning layer, the first latent layer of each
+    four run twice with its own cache (as the design's `weights_of` allows)."""
+    latent = {"heads": z["heads"], "dim": z["head"] - z["rot"], "rot_dim": z["rot"],
+              "vdim": z["vdim"], "kv_rank": z["rank"], "scale": z["head"] ** -0.5,
+              "rot": {"base": 10000.0, "dims": z["rot"],
+                      "scaling": {"factor": 4.0, "original": 1024, "fast": 32.0, "slow": 1.0}}}
+    lightning = {"heads": z["heads"], "dim": z["head"], "vdim": z["vdim"],
+                 "decay": [1.0 - 2.0 ** -(3 + 5 * h / max(z["heads"] - 1, 1)) for h in range(z["heads"])]}
+    mlp = {"kind": "dense", "ff": z["ff"]}
+    layers = []
+    for i in range(z["layers"]):
+        if i % 4 == 0:
+            layers.append({"type": "lightning", "mixer": lightning, "mlp": mlp})
+        elif i % 4 == 2:
+            layers.append({"type": "latent_attention", "mixer": latent, "mlp": mlp, "weights_of": i - 1})
+        else:
+            layers.append({"type": "latent_attention", "mixer": latent, "mlp": mlp})
+    return {"architecture": "Getodra", "vocab": z["vocab"], "width": z["width"],
+            "max_positions": z["positions"], "norm": {"eps": 1e-5}, "canon": {"taps": 4},
+            "layers": layers}
+
+
+def dense_config(z: dict) -> dict:
+    """The closest model the engine had before: pre-norm blocks of rotary attention (as many
+    heads of the same size, each with keys and values of its own) and a gated feed-forward."""
+    return dict(CONFIG_C, num_hidden_layers=z["layers"], hidden_size=z["width"],
+                num_attention_heads=z["heads"], num_key_value_heads=z["heads"], head_dim=z["head"],
+                intermediate_size=z["ff"], num_experts=0, num_experts_per_tok=0,
+                moe_intermediate_size=0, shared_expert_intermediate_size=0, vocab_size=z["vocab"],
+                hidden_act="gelu_pytorch_tanh")
+
+
+def designs_scenario(args) -> int:
+    import torch
+    from ninfer_amd import Chunk, EngineOptions, random_model
+
+    gen = torch.Generator().manual_seed(11)
+    out = {"metric": "prefill and decode throughput, Getodra beside a dense model of equal size",
+           "unit": "tok/s", "n_gpus": 1, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+           "data": "synthetic", "sizes": {}}
+    for size in args.sizes.split(","):
+        z = DESIGN_SIZES[size]
+        ctx = z["positions"]
+        row = {"shape": z}
+        for name, raw in (("getodra", getodra_config(z)), ("dense", dense_config(z))):
+            opt = EngineOptions(dtype=args.dtype, max_context=ctx, prefill_chunk=2048,
+                                num_sequences=64, page_size=16, use_graph=args.graph)
+            runner = random_model(raw, 99, opt)
+            for pools in runner.cache.pools.values():
+                for pool in pools.values():
+                    pool.normal_()
+            res = {}
+            for T in (512, 2048):
+                toks = torch.randint(0, z["vocab"], (T,), generator=gen).tolist()
+                times = []
+                for _ in range(5):
+                    s = runner.open()
+                    torch.cuda.synchronize()
+                    t = time.perf_counter()
+                    runner.step([Chunk(s, toks, [T - 1])])
+                    torch.cuda.synchronize()
+                    times.append(time.perf_counter() - t)
+                    runner.close(s)
+                dt = sorted(times[2:])[1]
+                res[f"prefill_{T}"] = {"tok_s": round(T / dt, 1), "ms": round(dt * 1e3, 3)}
+            steps, warm = max(8, args.steps // 2), 4
+            for batch in (1, 8, 64):
+                start = ctx - steps - warm - 1
+                slots = [runner.open() for _ in range(batch)]
+                for s in slots:
+                    runner.cache.reserve(s, start)
+                    runner.cache.commit(s, start)
+                toks = torch.randint(0, z["vocab"], (batch,), generator=gen).tolist()
+                for i in range(steps + warm):
+                    if i == warm:
+                        torch.cuda.synchronize()
+                        t = time.perf_counter()
+                    runner.step([Chunk(s, [tk], [0]) for s, tk in zip(slots, toks)])
+                torch.cuda.synchronize()
+                dt = (time.perf_counter() - t) / steps
+                for s in slots:
+                    runner.close(s)
+                res[f"decode_b{batch}_ctx{ctx}"] = {"tok_s": round(batch / dt, 1),
+                                                    "ms_per_step": round(dt * 1e3, 4)}
+            res["kv_bytes_per_token"] = runner.cache.kv_bytes_per_token(2 if args.dtype == "bfloat16" else 4)
+            res["state_bytes_per_request"] = runner.cache.state_bytes_per_request()
+            row[name] = res
+            print(f"[bench] {size} {name}: {json.dumps(res)}", file=sys.stderr, flush=True)
+            runner.release()
+            del runner
+            torch.cuda.empty_cache()
+        out["sizes"][size] = row
+    print(json.dumps(out), flush=True)
     return 0
 
 

@@ -16,6 +16,16 @@
 //                    row's position alone. The head's output may be multiplied by
 //                    sigmoid(gate[row, head]).
 //
+//   latent_attention_tile (bfloat16, matrix cores): a block of four waves owns 32 rows of
+//                    (token, head) pairs of one request, all of which read the same cached
+//                    rows. Keys come in tiles of 64 through LDS as they lie in the cache
+//                    ([key][numbers]); S = Q' K^T and O += P V run on v_mfma_f32_32x32x16_bf16,
+//                    the softmax between them in 32-bit on eight lanes per row. The value
+//                    operand needs eight keys of one column per lane and takes them from
+//                    the tile by eight two-byte LDS reads. The keys of long contexts are cut
+//                    into chunks over several blocks whose partial sums a second kernel
+//                    merges (steps of few rows would otherwise leave most of the GPU idle).
+//
 // The rotation turns pair (i, i + n/2) of the first n = rot_n numbers of the rotated part by
 // pos * freq[i]; cosine and sine are multiplied by `magnitude` (1 without a scaled table).
 // Norm, angles, scores, softmax and the value sum are 32-bit.
@@ -36,6 +46,13 @@ struct LatentArgs {
   const int* block_table;   // [S, bt_stride]
   const int* positions;     // [T]
   const int* row_seq;       // [T]
+  const int* seq_row_start; // [S + 1] (the matrix-core kernel: rows of each request)
+  const int* seq_pos0;      // [S] position of each request's first row
+  float* workspace;         // partial sums of contexts cut into chunks, or null
+  long long workspace_floats;
+  int S;
+  int max_kv_len;           // host-side bound that sizes the chunks
+  int force_plain;          // tests: the plain kernel whatever the shape
   int dkv_stride;
   int gate_stride;
   int bt_stride;
@@ -182,6 +199,9 @@ __global__ __launch_bounds__(64) void latent_attention_kernel(LatentArgs a) {
   }
 }
 
+static bool latent_tile_takes(const LatentArgs& a);
+static int latent_attention_tile(const LatentArgs& a, hipStream_t stream);
+
 static int latent_check(const LatentArgs& a, const char* who) {
   NINFER_REQUIRE(a.T > 0 && a.Hq > 0 && a.R > 0 && a.rd >= 0 && a.dim >= 0,
                  "%s: T=%d heads=%d latent=%d rotated=%d unrotated=%d", who, a.T, a.Hq, a.R, a.rd,
@@ -219,6 +239,7 @@ extern "C" int ninfer_latent_attention(const LatentArgs* a, hipStream_t stream) 
   NINFER_REQUIRE(a->R <= 64 * kLatentMaxPerLane, "latent_attention: latent size %d exceeds %d",
                  a->R, 64 * kLatentMaxPerLane);
   NINFER_REQUIRE(a->scale > 0.f, "latent_attention: scale %g must be positive", (double)a->scale);
+  if (latent_tile_takes(*a)) return latent_attention_tile(*a, stream);
   const dim3 grid(a->T, a->Hq);
   const size_t lds = (size_t)(a->R + a->rd + 64) * sizeof(float) + 64 * sizeof(int64_t);
   NINFER_REQUIRE(lds <= 64 * 1024, "latent_attention: a query of %d numbers does not fit",
@@ -229,4 +250,355 @@ extern "C" int ninfer_latent_attention(const LatentArgs* a, hipStream_t stream) 
     latent_attention_kernel<bf16><<<grid, 64, lds, stream>>>(*a);
   NINFER_LAUNCH_CHECK();
   return 0;
+}
+
+// ---- the matrix-core kernel ------------------------------------------------------------------
+namespace ninfer {
+
+typedef __bf16 lat_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float lat_f32x16 __attribute__((ext_vector_type(16)));
+
+constexpr int kLatRows = 32;      // (token, head) rows per block
+constexpr int kLatKeys = 64;      // keys per tile
+constexpr int kLatColTiles = 4;   // 32-column tiles of the output per wave: latent sizes up to 512
+
+struct LatentTilePlan {
+  int tiles;        // upper bound of row tiles over all requests
+  int n_chunks;     // key chunks per row tile
+  int chunk;        // keys per chunk (a multiple of 64)
+  int dkp;          // row length of Q in LDS (numbers)
+  int kstr;         // row length of a key in LDS (numbers)
+  int page_shift;
+  size_t lds;
+};
+
+static bool latent_tile_takes(const LatentArgs& a) {
+  const int Dk = a.R + a.rd;
+  return a.dtype == kBF16 && !a.force_plain && Dk % 8 == 0 && a.R <= 32 * 4 * kLatColTiles &&
+         (a.page_size & (a.page_size - 1)) == 0 && a.seq_row_start && a.seq_pos0 && a.S > 0 &&
+         ((uintptr_t)a.pool % 16 == 0);
+}
+
+static LatentTilePlan latent_tile_plan(const LatentArgs& a) {
+  LatentTilePlan p;
+  const int Dk = a.R + a.rd;
+  const int dk16 = (Dk + 15) / 16 * 16;
+  const int cols = (a.R + 31) / 32 * 32;
+  p.dkp = dk16 + 8;
+  p.kstr = (dk16 > cols ? dk16 : cols) + 8;
+  p.tiles = (int)(((int64_t)a.T * a.Hq + kLatRows - 1) / kLatRows) + a.S;
+  const int key_tiles = (a.max_kv_len + kLatKeys - 1) / kLatKeys;
+  int want = (2 * device_cu_count() + p.tiles - 1) / p.tiles;   // blocks enough for two a CU
+  if (want > key_tiles) want = key_tiles;
+  if (want < 1) want = 1;
+  const int tiles_per_chunk = (key_tiles + want - 1) / want;
+  p.chunk = tiles_per_chunk * kLatKeys;
+  p.n_chunks = (key_tiles + tiles_per_chunk - 1) / tiles_per_chunk;
+  p.page_shift = 0;
+  while ((1 << p.page_shift) < a.page_size) ++p.page_shift;
+  p.lds = (size_t)kLatRows * p.dkp * 2 + (size_t)kLatKeys * p.kstr * 2 +
+          2 * kLatRows * kLatKeys * 4 + kLatRows * (kLatKeys + 8) * 2 + 3 * kLatRows * 4;
+  return p;
+}
+
+static int64_t latent_tile_workspace_floats(const LatentArgs& a, const LatentTilePlan& p) {
+  return p.n_chunks > 1 ? (int64_t)a.T * a.Hq * p.n_chunks * (a.R + 2) : 0;
+}
+
+__global__ __launch_bounds__(256) void latent_attention_tile_kernel(LatentArgs a, LatentTilePlan pl) {
+  extern __shared__ float smem[];
+  const int Dk = a.R + a.rd, R = a.R, H = a.Hq;
+  __bf16* Qs = (__bf16*)smem;                                   // [32][dkp]
+  __bf16* Ks = Qs + kLatRows * pl.dkp;                          // [64][kstr]
+  float* Sp = (float*)(Ks + kLatKeys * pl.kstr);                // [2][32][64]
+  __bf16* Ps = (__bf16*)(Sp + 2 * kLatRows * kLatKeys);         // [32][72]
+  float* alpha_s = (float*)(Ps + kLatRows * (kLatKeys + 8));    // [32], then m [32], l [32]
+  float* m_s = alpha_s + kLatRows;
+  float* l_s = m_s + kLatRows;
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int lr = lane & 31, lk = lane >> 5;
+
+  // which request and which of its row tiles is this block's?
+  int s = -1, lt = 0;
+  {
+    int left = blockIdx.x;
+    for (int i = 0; i < a.S; ++i) {
+      const int n = (a.seq_row_start[i + 1] - a.seq_row_start[i]) * H;
+      const int nt = (n + kLatRows - 1) / kLatRows;
+      if (left < nt) {
+        s = i;
+        lt = left;
+        break;
+      }
+      left -= nt;
+    }
+  }
+  if (s < 0) return;
+  const int chunk_id = blockIdx.y;
+  const int row0 = a.seq_row_start[s];
+  const int n_flat = (a.seq_row_start[s + 1] - row0) * H;
+  const int pos0 = a.seq_pos0[s];
+  const int f0 = lt * kLatRows;                          // first flattened row of the tile
+  const int rows_here = min(kLatRows, n_flat - f0);
+  const int tok_first = f0 / H, tok_last = (f0 + rows_here - 1) / H;
+  const int pos_last = pos0 + tok_last;
+  const int lo_first = a.window > 0 ? max(0, pos0 + tok_first - a.window + 1) : 0;
+  // this block's keys: its chunk of the context, cut to what its rows can see
+  const int k_begin = max(chunk_id * pl.chunk, lo_first / kLatKeys * kLatKeys);
+  const int k_end = min((chunk_id + 1) * pl.chunk, pos_last + 1);
+  const int* bt = a.block_table + (int64_t)s * a.bt_stride;
+  const __bf16* pool = (const __bf16*)a.pool;
+
+  // Q' of the tile's rows as bfloat16, zeros in rows and columns that are not there
+  for (int e = tid; e < kLatRows * pl.dkp; e += 256) {
+    const int i = e / pl.dkp, d = e % pl.dkp;
+    float v = 0.f;
+    if (i < rows_here && d < Dk) {
+      const int f = f0 + i;
+      v = a.q_abs[((int64_t)(row0 + f / H) * H + f % H) * Dk + d];
+    }
+    Qs[e] = (__bf16)v;
+  }
+  for (int e = tid; e < kLatKeys * pl.kstr; e += 256) Ks[e] = (__bf16)0.f;   // the pads stay zero
+  __syncthreads();
+
+  // softmax threads: row tid / 8, keys 8 (tid % 8) .. + 7 of a tile
+  const int sm_row = tid >> 3, sm_part = tid & 7;
+  int sm_pos = -1, sm_lo = 0;
+  if (sm_row < rows_here) {
+    sm_pos = pos0 + (f0 + sm_row) / H;
+    sm_lo = a.window > 0 ? max(0, sm_pos - a.window + 1) : 0;
+  }
+  float m_run = -INFINITY, l_run = 0.f;
+
+  lat_f32x16 acc[kLatColTiles];
+#pragma unroll
+  for (int c = 0; c < kLatColTiles; ++c)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[c][i] = 0.f;
+  const int n_ct = (R + 31) / 32;
+  const int ct_per_wave = (n_ct + 3) / 4;
+  const int ksteps = (Dk + 15) / 16;
+  const int ks_half = (ksteps + 1) / 2;
+  const int cpr = Dk / 8;   // 16-byte pieces of a cached row
+
+  for (int kt = k_begin; kt < k_end; kt += kLatKeys) {
+    // 1. the tile's keys into LDS as they lie in their pages
+    for (int e = tid; e < kLatKeys * cpr; e += 256) {
+      const int j = e / cpr, c = e % cpr;
+      const int kp = kt + j;
+      lat_bf16x8 v;
+#pragma unroll
+      for (int x = 0; x < 8; ++x) v[x] = (__bf16)0.f;
+      if (kp <= pos_last) {
+        const int page = bt[kp >> pl.page_shift];
+        if (page >= 0)
+          v = *(const lat_bf16x8*)(pool + ((int64_t)page * a.page_size + (kp & (a.page_size - 1))) * Dk + 8 * c);
+      }
+      *(lat_bf16x8*)(Ks + j * pl.kstr + 8 * c) = v;
+    }
+    __syncthreads();
+    // 2. S = Q' K^T: wave w meets keys 32 (w & 1) .. + 31 over one half of the numbers
+    {
+      const int n = w & 1, kh = w >> 1;
+      lat_f32x16 sacc;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) sacc[i] = 0.f;
+      const int s_lo = kh ? ks_half : 0, s_hi = kh ? ksteps : ks_half;
+      const __bf16* qrow = Qs + lr * pl.dkp + 8 * lk;
+      const __bf16* krow = Ks + (32 * n + lr) * pl.kstr + 8 * lk;
+      for (int st = s_lo; st < s_hi; ++st) {
+        const lat_bf16x8 qf = *(const lat_bf16x8*)(qrow + 16 * st);
+        const lat_bf16x8 kf = *(const lat_bf16x8*)(krow + 16 * st);
+        sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qf, kf, sacc, 0, 0, 0);
+      }
+      // the lane holds key 32 n + lr for rows 8 q + 4 lk + r in register 4 q + r
+      float* sp = Sp + kh * kLatRows * kLatKeys + 32 * n + lr;
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) sp[(8 * q + 4 * lk + r) * kLatKeys] = sacc[4 * q + r];
+    }
+    __syncthreads();
+    // 3. softmax of the tile, 32-bit: eight lanes per row
+    {
+      float sv[8];
+      float mx = -INFINITY;
+#pragma unroll
+      for (int x = 0; x < 8; ++x) {
+        const int j = 8 * sm_part + x;
+        const int kp = kt + j;
+        const float v = (Sp[sm_row * kLatKeys + j] + Sp[kLatRows * kLatKeys + sm_row * kLatKeys + j]) * a.scale;
+        const bool see = kp <= sm_pos && kp >= sm_lo;
+        sv[x] = see ? v : -INFINITY;
+        mx = fmaxf(mx, sv[x]);
+      }
+      mx = fmaxf(mx, __shfl_xor(mx, 1, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 2, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 4, 64));
+      const float m_new = fmaxf(m_run, mx);
+      float al = 1.f, sum = 0.f;
+      lat_bf16x8 pv;
+      if (m_new == -INFINITY) {   // nothing seen so far
+#pragma unroll
+        for (int x = 0; x < 8; ++x) pv[x] = (__bf16)0.f;
+      } else {
+        al = expf(m_run - m_new);   // 0 while m_run is minus infinity
+#pragma unroll
+        for (int x = 0; x < 8; ++x) {
+          const float p = expf(sv[x] - m_new);
+          pv[x] = (__bf16)p;
+          sum += p;
+        }
+      }
+      sum += __shfl_xor(sum, 1, 64);
+      sum += __shfl_xor(sum, 2, 64);
+      sum += __shfl_xor(sum, 4, 64);
+      l_run = l_run * al + sum;
+      m_run = m_new;
+      *(lat_bf16x8*)(Ps + sm_row * (kLatKeys + 8) + 8 * sm_part) = pv;
+      if (sm_part == 0) alpha_s[sm_row] = al;
+    }
+    __syncthreads();
+    // 4. O = O alpha + P V on this wave's column tiles
+    {
+      const float al = alpha_s[lr];   // every register of the lane belongs to row lr
+      lat_bf16x8 pf[4];
+#pragma unroll
+      for (int st = 0; st < 4; ++st)
+        pf[st] = *(const lat_bf16x8*)(Ps + lr * (kLatKeys + 8) + 16 * st + 8 * lk);
+#pragma unroll
+      for (int c = 0; c < kLatColTiles; ++c) {
+        const int ct = w * ct_per_wave + c;
+        if (c < ct_per_wave && ct < n_ct) {
+#pragma unroll
+          for (int i = 0; i < 16; ++i) acc[c][i] *= al;
+          const __bf16* vcol = Ks + 32 * ct + lr;
+#pragma unroll
+          for (int st = 0; st < 4; ++st) {
+            lat_bf16x8 vf;
+#pragma unroll
+            for (int x = 0; x < 8; ++x) vf[x] = vcol[(16 * st + 8 * lk + x) * pl.kstr];
+            // A = V^T: lane holds column 32 ct + lr for 8 keys; B = P^T: row lr for the same keys
+            acc[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[st], acc[c], 0, 0, 0);
+          }
+        }
+      }
+    }
+    __syncthreads();
+  }
+
+  if (sm_part == 0) {
+    m_s[sm_row] = m_run;
+    l_s[sm_row] = l_run;
+  }
+  __syncthreads();
+  // With A = V^T and B = P^T the lane holds row lr of the tile (a (token, head) pair) and the
+  // columns 32 ct + 8 q + 4 lk + r in register 4 q + r.
+  if (lr < rows_here) {
+    const int f = f0 + lr;
+    const int t = row0 + f / H, h = f % H;
+    const float l = l_s[lr], m = m_s[lr];
+    if (pl.n_chunks == 1) {
+      float inv = l > 0.f ? 1.f / l : 0.f;
+      if (a.gate) {
+        const float g = __bfloat162float(((const bf16*)a.gate)[(int64_t)t * a.gate_stride + h]);
+        inv *= 1.f / (1.f + expf(-g));
+      }
+      __bf16* orow = (__bf16*)a.out + ((int64_t)t * H + h) * R;
+#pragma unroll
+      for (int c = 0; c < kLatColTiles; ++c) {
+        const int ct = w * ct_per_wave + c;
+        if (c < ct_per_wave && ct < n_ct) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const int d = 32 * ct + 8 * q + 4 * lk + r;
+              if (d < R) orow[d] = (__bf16)(acc[c][4 * q + r] * inv);
+            }
+        }
+      }
+    } else {
+      float* part = a.workspace + (((int64_t)t * H + h) * pl.n_chunks + chunk_id) * (R + 2);
+      if (w == 0 && lk == 0) {
+        part[R] = m;
+        part[R + 1] = l;
+      }
+#pragma unroll
+      for (int c = 0; c < kLatColTiles; ++c) {
+        const int ct = w * ct_per_wave + c;
+        if (c < ct_per_wave && ct < n_ct) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const int d = 32 * ct + 8 * q + 4 * lk + r;
+              if (d < R) part[d] = acc[c][4 * q + r];
+            }
+        }
+      }
+    }
+  }
+}
+
+// out[t, h] = sum_c e^(m_c - M) O_c / sum_c e^(m_c - M) l_c over the chunks that saw keys.
+__global__ void latent_attention_merge_kernel(LatentArgs a, int n_chunks) {
+  const int64_t th = blockIdx.x;
+  const int R = a.R;
+  const float* part = a.workspace + th * n_chunks * (R + 2);
+  float M = -INFINITY;
+  for (int c = 0; c < n_chunks; ++c) M = fmaxf(M, part[c * (R + 2) + R]);
+  float L = 0.f;
+  for (int c = 0; c < n_chunks; ++c) {
+    const float m = part[c * (R + 2) + R];
+    if (m > -INFINITY) L += expf(m - M) * part[c * (R + 2) + R + 1];
+  }
+  float inv = L > 0.f ? 1.f / L : 0.f;
+  if (a.gate) {
+    const int t = (int)(th / a.Hq), h = (int)(th % a.Hq);
+    const float g = __bfloat162float(((const bf16*)a.gate)[(int64_t)t * a.gate_stride + h]);
+    inv *= 1.f / (1.f + expf(-g));
+  }
+  __bf16* orow = (__bf16*)a.out + th * R;
+  for (int d = threadIdx.x; d < R; d += blockDim.x) {
+    float o = 0.f;
+    for (int c = 0; c < n_chunks; ++c) {
+      const float m = part[c * (R + 2) + R];
+      if (m > -INFINITY) o += expf(m - M) * part[c * (R + 2) + d];
+    }
+    orow[d] = (__bf16)(o * inv);
+  }
+}
+
+static int latent_attention_tile(const LatentArgs& a, hipStream_t stream) {
+  const LatentTilePlan p = latent_tile_plan(a);
+  NINFER_REQUIRE(p.lds <= 160 * 1024, "latent_attention: rows of %d numbers do not fit the LDS",
+                 a.R + a.rd);
+  const int64_t need = latent_tile_workspace_floats(a, p);
+  NINFER_REQUIRE(need == 0 || (a.workspace && a.workspace_floats >= need),
+                 "latent_attention: the workspace holds %lld floats, %lld are needed",
+                 (long long)a.workspace_floats, (long long)need);
+  auto kern = latent_attention_tile_kernel;
+  if (p.lds > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       (int)p.lds);
+    if (e != hipSuccess) return set_error(-2, "latent_attention: cannot get %zu bytes of LDS", p.lds);
+  }
+  kern<<<dim3(p.tiles, p.n_chunks), 256, p.lds, stream>>>(a, p);
+  NINFER_LAUNCH_CHECK();
+  if (p.n_chunks > 1) {
+    const int block = a.R >= 256 ? 256 : (a.R + 63) / 64 * 64;
+    latent_attention_merge_kernel<<<(unsigned)((int64_t)a.T * a.Hq), block, 0, stream>>>(a, p.n_chunks);
+    NINFER_LAUNCH_CHECK();
+  }
+  return 0;
+}
+
+}  // namespace ninfer
+
+// 32-bit floats of workspace that a step of this shape needs (0: none).
+extern "C" long long ninfer_latent_attention_workspace_floats(const ninfer::LatentArgs* a) {
+  if (!ninfer::latent_tile_takes(*a)) return 0;
+  return ninfer::latent_tile_workspace_floats(*a, ninfer::latent_tile_plan(*a));
 }

@@ -93,7 +93,11 @@ class _LatentArgs(ctypes.Structure):
                 ("pool", ctypes.c_void_p), ("out", ctypes.c_void_p), ("gate", ctypes.c_void_p),
                 ("norm_w", ctypes.c_void_p), ("freq", ctypes.c_void_p),
                 ("block_table", ctypes.c_void_p), ("positions", ctypes.c_void_p),
-                ("row_seq", ctypes.c_void_p), ("dkv_stride", ctypes.c_int),
+                ("row_seq", ctypes.c_void_p), ("seq_row_start", ctypes.c_void_p),
+                ("seq_pos0", ctypes.c_void_p), ("workspace", ctypes.c_void_p),
+                ("workspace_floats", ctypes.c_longlong), ("S", ctypes.c_int),
+                ("max_kv_len", ctypes.c_int), ("force_plain", ctypes.c_int),
+                ("dkv_stride", ctypes.c_int),
                 ("gate_stride", ctypes.c_int), ("bt_stride", ctypes.c_int), ("T", ctypes.c_int),
                 ("Hq", ctypes.c_int), ("dim", ctypes.c_int), ("R", ctypes.c_int),
                 ("rd", ctypes.c_int), ("rot_n", ctypes.c_int), ("page_size", ctypes.c_int),
@@ -203,6 +207,7 @@ class HipOps:
         self.lib.ninfer_event_create.restype = ctypes.c_void_p
         self.lib.ninfer_stream_after.argtypes = [ctypes.c_void_p] * 3
         self.lib.ninfer_sample_few_places.restype = ctypes.c_longlong
+        self.lib.ninfer_latent_attention_workspace_floats.restype = ctypes.c_longlong
         self.force_generic = False  # tests: run the plain kernels whatever the shape
         self._device_index = None   # the one GPU's index, asked for at the first launch
         self._held = None           # products held back inside `together()`
@@ -951,6 +956,8 @@ class HipOps:
         a = _LatentArgs()
         a.pool, a.block_table = pool.data_ptr(), block_table.data_ptr()
         a.positions, a.row_seq = ctx.positions.data_ptr(), ctx.row_seq.data_ptr()
+        a.seq_row_start, a.seq_pos0 = ctx.seq_row_start.data_ptr(), ctx.seq_pos0.data_ptr()
+        a.S, a.max_kv_len, a.force_plain = ctx.S, ctx.max_kv_len, 1 if self.force_generic else 0
         a.bt_stride, a.T, a.Hq, a.dim, a.R, a.rd, a.rot_n = \
             block_table.shape[1], ctx.T, heads, dim, rank, rot_dim, rot_n
         a.page_size, a.dtype = page_size, _DT[dtype]
@@ -1004,7 +1011,22 @@ class HipOps:
                   and gate.stride(1) == 1, "latent_attention: the gate must be [T, heads] columns")
             a.gate = gate.data_ptr()
             a.gate_stride = gate.stride(0) if t > 1 else max(heads, gate.stride(0))
+        need = int(self.lib.ninfer_latent_attention_workspace_floats(ctypes.byref(a)))
+        if need:   # contexts cut into chunks: partial sums, merged by a second kernel
+            ws = self._workspace(need, q_abs.device)
+            a.workspace, a.workspace_floats = ws.data_ptr(), ws.numel()
         self._ok(self.lib.ninfer_latent_attention(ctypes.byref(a), self._stream()))
+
+    def _workspace(self, floats: int, device) -> torch.Tensor:
+        """The attention kernels' 32-bit scratch, grown when a step needs more. A captured graph
+        may hold the address of the one it was recorded with: an outgrown one is kept, never
+        given back, and growth at least doubles, which bounds what is kept."""
+        if self._attn_ws is None or self._attn_ws.numel() < floats:
+            if self._attn_ws is not None:
+                self._outgrown.append(self._attn_ws)
+                floats = max(floats, 2 * self._attn_ws.numel())
+            self._attn_ws = torch.empty(floats, dtype=torch.float32, device=device)
+        return self._attn_ws
 
     def head_index(self, ctx, heads):
         """(offsets [heads + 1], index [T * heads]) for products that every head runs with

@@ -230,6 +230,33 @@ def test_latent_attention_rows(ops, dtype, heads, rank, rd, ps):
     assert rel_err(got, want) < (1e-5 if dtype == torch.float32 else 6e-3)
 
 
+@pytest.mark.parametrize("heads,rank,rd", [(16, 64, 16), (5, 200, 24)])
+def test_latent_attention_whole_prompt_on_matrix_cores(ops, heads, rank, rd):
+    """A prompt long enough that the bfloat16 kernel walks each block's keys in one piece
+    (shorter steps cut the keys into chunks and merge), against the plain kernel and
+    against the softmax written out."""
+    n, ps = 1100, 16
+    ctx, pool, table, q, cached = _latent_case(ops, torch.bfloat16, heads, rank, rd, ps, [n], [n], seed=rank)
+    keys = cached[0].double()
+    want = torch.zeros(n, heads, rank, dtype=torch.float64)
+    mask = torch.tril(torch.ones(n, n, dtype=torch.bool))
+    for h in range(heads):
+        s = (q[:, h].double() @ keys.T * 0.3).masked_fill(~mask, float("-inf"))
+        want[:, h] = torch.softmax(s, -1) @ keys[:, :rank]
+    outs = []
+    for plain in (False, True):
+        ops.force_generic = plain
+        try:
+            out = torch.empty(n, heads * rank, dtype=torch.bfloat16, device=DEV)
+            ops.latent_attention(q.to(DEV), pool.to(torch.bfloat16).to(DEV), table.to(DEV), ctx, heads,
+                                 rank, rd, ps, 0.3, out)
+        finally:
+            ops.force_generic = False
+        outs.append(out.float().cpu().reshape(n, heads, rank))
+        assert rel_err(outs[-1], want) < 8e-3
+    assert rel_err(outs[0][:3], want[:3]) < 8e-3 and rel_err(outs[0][-1], want[-1]) < 8e-3
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("where", [0, 1, 15, 16, 63, 64, 300, 498])
 def test_latent_attention_finds_one_key(ops, dtype, where):
@@ -380,8 +407,9 @@ def check_logits(case, dtype, got, what):
             (8 * 2.0 ** -15, 8 * 2.0 ** -15, 16 * 2.0 ** -15, 3e-6)
         e50 = err.median().item()
         e90 = err.kthvalue(max(1, int(0.9 * len(err)))).values.item()
-        assert e50 <= max(f50 * n50, floor), f"{who}: median row error {e50:.2e} (disturbance {n50:.2e})"
-        assert e90 <= max(f90 * n90, floor), f"{who}: ninth decile {e90:.2e} (disturbance {n90:.2e})"
+        if len(err) >= 20:   # (deciles of a handful of rows say little)
+            assert e50 <= max(f50 * n50, floor), f"{who}: median row error {e50:.2e} (disturbance {n50:.2e})"
+            assert e90 <= max(f90 * n90, floor), f"{who}: ninth decile {e90:.2e} (disturbance {n90:.2e})"
         assert err.max().item() <= max(fmax * nmax, 4 * floor), \
             f"{who}: row {err.argmax()} is off by {err.max():.2e} (disturbance {nmax:.2e})"
 
