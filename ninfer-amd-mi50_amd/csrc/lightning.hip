@@ -114,3 +114,230 @@ extern "C" int ninfer_lightning_attention(const void* qkv, int stride, int q_off
   NINFER_LAUNCH_CHECK();
   return 0;
 }
+
+// ---- prompt portions in chunks, on the 32-bit matrix instruction --------------------------------
+//
+// For the rows i = 0 .. L - 1 of a chunk (L <= 64) with the state S before it:
+//
+//   o_i = sum_{j <= i} d^(i - j) (q_i . k_j) v_j  +  d^(i + 1) S^T q_i
+//   S' = d^L S + sum_j d^(L - 1 - j) k_j v_j^T
+//
+// which is the recurrence written out; all powers of the decay have exponents >= 0, so nothing
+// grows. Every product runs on v_mfma_f32_32x32x2_f32: q, k, v (silu of the projections), the
+// decays and the state enter in 32-bit and are never rounded to a shorter type. A block owns
+// one (request, head, 32 value columns): the chunks of a request follow each other in it, and
+// the value columns of a head are independent, which gives the launch heads x vdim / 32 blocks
+// per request. Waves 0 and 1 form the chunk's outputs, waves 2 and 3 carry the state in their
+// accumulators and hand a copy to the others through LDS.
+namespace ninfer {
+
+typedef float lt_f32x16 __attribute__((ext_vector_type(16)));
+constexpr int kLtChunk = 64;
+constexpr int kLtStateTiles = 4;   // 32-row tiles of the state per carrying wave: dim up to 256
+
+__device__ __forceinline__ float decay_pow(float log2d, int n) {
+  return n == 0 ? 1.f : exp2f((float)n * log2d);   // (a decay of 0 has log2 -inf: 0 * -inf is no number)
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void lightning_chunk_kernel(
+    const T* __restrict__ qkv, int stride, int q_off, int k_off, int v_off,
+    const float* __restrict__ decay, float* __restrict__ state, int64_t state_stride,
+    float* __restrict__ out, const int* __restrict__ seq_row_start,
+    const int* __restrict__ seq_slots, int H, int dim, int vdim) {
+  extern __shared__ float smem[];
+  const int qs = dim + 1;                 // row length of q and k in LDS (odd: column reads spread)
+  float* Qs = smem;                       // [64][dim + 1]
+  float* Ks = Qs + kLtChunk * qs;         // [64][dim + 1]
+  float* Vs = Ks + kLtChunk * qs;         // [64][33]
+  float* As = Vs + kLtChunk * 33;         // [64][65]
+  float* Ss = As + kLtChunk * 65;         // [dim32][33]
+  const int s = blockIdx.x, h = blockIdx.y, c0 = 32 * blockIdx.z;
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, lr = lane & 31, lk = lane >> 5;
+  const int r0 = seq_row_start[s], n = seq_row_start[s + 1] - r0;
+  const int dim32 = (dim + 31) / 32 * 32;
+  const int d_tiles = dim32 / 32;
+  float* st = state + (int64_t)seq_slots[s] * state_stride + (int64_t)h * dim * vdim;
+  const float dec = decay[h];
+  const float log2d = log2f(dec);
+  const bool col_ok = c0 + lr < vdim;
+
+  // the state: in the accumulators of waves 2 and 3 (tiles w - 2, w, ...), a copy in LDS
+  lt_f32x16 sacc[kLtStateTiles];
+#pragma unroll
+  for (int x = 0; x < kLtStateTiles; ++x)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) sacc[x][i] = 0.f;
+  for (int e = tid; e < dim32 * 33; e += 256) {
+    const int d = e / 33, c = e % 33;
+    Ss[e] = (d < dim && c < 32 && c0 + c < vdim) ? st[(int64_t)d * vdim + c0 + c] : 0.f;
+  }
+  __syncthreads();
+  if (w >= 2) {
+#pragma unroll
+    for (int x = 0; x < kLtStateTiles; ++x) {
+      const int dt = (w - 2) + 2 * x;
+      if (dt < d_tiles) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) sacc[x][4 * q + r] = Ss[(32 * dt + 8 * q + 4 * lk + r) * 33 + lr];
+      }
+    }
+  }
+
+  for (int i0 = 0; i0 < n; i0 += kLtChunk) {
+    const int L = min(kLtChunk, n - i0);
+    // 1. the chunk's q, k (all of the head's numbers) and this block's value columns
+    for (int e = tid; e < kLtChunk * dim; e += 256) {
+      const int i = e / dim, d = e % dim;
+      float qv = 0.f, kv = 0.f;
+      if (i < L) {
+        const T* row = qkv + (int64_t)(r0 + i0 + i) * stride;
+        qv = silu_f(to_f32(row[q_off + h * dim + d]));
+        kv = silu_f(to_f32(row[k_off + h * dim + d]));
+      }
+      Qs[i * qs + d] = qv;
+      Ks[i * qs + d] = kv;
+    }
+    for (int e = tid; e < kLtChunk * 32; e += 256) {
+      const int i = e >> 5, c = e & 31;
+      float vv = 0.f;
+      if (i < L && c0 + c < vdim)
+        vv = silu_f(to_f32(qkv[(int64_t)(r0 + i0 + i) * stride + v_off + h * vdim + c0 + c]));
+      Vs[i * 33 + c] = vv;
+    }
+    __syncthreads();   // (also: the state's copy in LDS is the one before this chunk)
+    // 2. A[i][j] = d^(i - j) q_i . k_j for j <= i: wave w has rows 32 (w / 2).., keys 32 (w % 2)..
+    {
+      const int mi = w >> 1, nj = w & 1;
+      lt_f32x16 a;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) a[i] = 0.f;
+      if (nj <= mi) {
+        const float* qrow = Qs + (32 * mi + lr) * qs + lk;
+        const float* krow = Ks + (32 * nj + lr) * qs + lk;
+        for (int d = 0; d + 1 < dim + 1 && d < dim; d += 2) {
+          const float qa = (d + lk < dim) ? qrow[d] : 0.f;
+          const float kb = (d + lk < dim) ? krow[d] : 0.f;
+          a = __builtin_amdgcn_mfma_f32_32x32x2f32(qa, kb, a, 0, 0, 0);
+        }
+      }
+      const int j = 32 * nj + lr;
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int i = 32 * mi + 8 * q + 4 * lk + r;
+          As[i * 65 + j] = j <= i ? a[4 * q + r] * decay_pow(log2d, i - j) : 0.f;
+        }
+    }
+    __syncthreads();
+    // 3. waves 0, 1: the outputs of rows 32 w ..; waves 2, 3: the state after the chunk
+    if (w < 2) {
+      lt_f32x16 o;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) o[i] = 0.f;
+      const int row = 32 * w + lr;
+      const float* arow = As + row * 65 + lk;
+      for (int j = 0; j < 32 * (w + 1); j += 2)
+        o = __builtin_amdgcn_mfma_f32_32x32x2f32(arow[j], Vs[(j + lk) * 33 + lr], o, 0, 0, 0);
+      const float carry = decay_pow(log2d, row + 1);
+      const float* qrow = Qs + row * qs + lk;
+      for (int d = 0; d < dim; d += 2) {
+        const float qa = (d + lk < dim) ? qrow[d] * carry : 0.f;
+        o = __builtin_amdgcn_mfma_f32_32x32x2f32(qa, Ss[(d + lk) * 33 + lr], o, 0, 0, 0);
+      }
+      if (col_ok) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int i = 32 * w + 8 * q + 4 * lk + r;
+            if (i < L) out[((int64_t)(r0 + i0 + i) * H + h) * vdim + c0 + lr] = o[4 * q + r];
+          }
+      }
+    } else {
+      const float whole = decay_pow(log2d, L);
+#pragma unroll
+      for (int x = 0; x < kLtStateTiles; ++x) {
+        const int dt = (w - 2) + 2 * x;
+        if (dt < d_tiles) {
+#pragma unroll
+          for (int i = 0; i < 16; ++i) sacc[x][i] *= whole;
+          const int d = 32 * dt + lr;
+          for (int j = 0; j < kLtChunk; j += 2) {
+            const int jj = j + lk;
+            const float ka = (jj < L && d < dim) ? Ks[jj * qs + d] * decay_pow(log2d, L - 1 - jj) : 0.f;
+            sacc[x] = __builtin_amdgcn_mfma_f32_32x32x2f32(ka, Vs[jj * 33 + lr], sacc[x], 0, 0, 0);
+          }
+        }
+      }
+    }
+    __syncthreads();   // everyone has read the old copy of the state
+    if (w >= 2) {
+#pragma unroll
+      for (int x = 0; x < kLtStateTiles; ++x) {
+        const int dt = (w - 2) + 2 * x;
+        if (dt < d_tiles) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) Ss[(32 * dt + 8 * q + 4 * lk + r) * 33 + lr] = sacc[x][4 * q + r];
+        }
+      }
+    }
+    // (the barrier after the next chunk's loads publishes the copy; nothing reads it before)
+  }
+  if (w >= 2 && col_ok) {
+#pragma unroll
+    for (int x = 0; x < kLtStateTiles; ++x) {
+      const int dt = (w - 2) + 2 * x;
+      if (dt < d_tiles) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int d = 32 * dt + 8 * q + 4 * lk + r;
+            if (d < dim) st[(int64_t)d * vdim + c0 + lr] = sacc[x][4 * q + r];
+          }
+      }
+    }
+  }
+}
+
+static size_t lightning_chunk_lds(int dim) {
+  const int dim32 = (dim + 31) / 32 * 32;
+  return ((size_t)2 * kLtChunk * (dim + 1) + kLtChunk * 33 + kLtChunk * 65 + (size_t)dim32 * 33) * sizeof(float);
+}
+
+}  // namespace ninfer
+
+// The same as ninfer_lightning_attention for bfloat16 rows, chunk by chunk on the matrix cores:
+// for steps that bring prompt portions. Returns 1 (nothing launched) when the sizes do not fit.
+extern "C" int ninfer_lightning_attention_chunks(const void* qkv, int stride, int q_off, int k_off,
+                                                 int v_off, const float* decay, float* state,
+                                                 long long state_stride, float* out,
+                                                 const int* seq_row_start, const int* seq_slots,
+                                                 int T, int S, int H, int dim, int vdim, int dtype,
+                                                 hipStream_t stream) {
+  NINFER_REQUIRE(T > 0 && S > 0 && H > 0 && dim > 0 && vdim > 0,
+                 "lightning_attention: T=%d S=%d heads=%d dim=%d vdim=%d must be positive", T, S,
+                 H, dim, vdim);
+  NINFER_REQUIRE(state_stride >= (long long)H * dim * vdim,
+                 "lightning_attention: a request's state of %lld floats holds no %d x %d x %d",
+                 state_stride, H, dim, vdim);
+  const size_t lds = lightning_chunk_lds(dim);
+  if (dtype != kBF16 || dim > 64 * kLtStateTiles || lds > 160 * 1024) return 1;
+  auto kern = lightning_chunk_kernel<bf16>;
+  if (lds > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       (int)lds);
+    if (e != hipSuccess) return set_error(-2, "lightning_attention: cannot get %zu bytes of LDS", lds);
+  }
+  kern<<<dim3(S, H, (vdim + 31) / 32), 256, lds, stream>>>(
+      (const bf16*)qkv, stride, q_off, k_off, v_off, decay, state, state_stride, out,
+      seq_row_start, seq_slots, H, dim, vdim);
+  NINFER_LAUNCH_CHECK();
+  return 0;
+}

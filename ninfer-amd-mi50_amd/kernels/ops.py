@@ -230,6 +230,7 @@ class HipOps:
         # (65: a decode step of up to 64 rows takes the same kernels run eagerly and captured)
         self.beside_heavy_min_rows = 65
         self.beside_heavy_bytes = 256 << 20
+        self.lightning_chunk_min_rows = 8   # a step's longest portion from which lightning attention runs in chunks
         self.library_min_rows = 32  # dense bf16 products with more rows go to the library
         self.rows_kernel_max = 64   # ... unless the kernel for 33 to 64 rows takes them
         self.rows_kernel_features = (4096, 32768)   # (gemm_skinny_rows.hip: where it beats the library)
@@ -938,12 +939,22 @@ class HipOps:
         _need(state.is_cuda and state.dtype == torch.float32 and state.dim() == 2
               and state.stride(1) == 1 and state.shape[1] >= heads * dim * vdim,
               "lightning_attention: the state must be 32-bit rows of heads * dim * vdim numbers")
-        self._ok(self.lib.ninfer_lightning_attention(
-            ctypes.c_void_p(qkv.data_ptr()), qkv.shape[1], q_off, k_off, v_off,
-            ctypes.c_void_p(decay.data_ptr()), ctypes.c_void_p(state.data_ptr()),
-            ctypes.c_longlong(state.stride(0)), ctypes.c_void_p(out.data_ptr()),
-            ctypes.c_void_p(ctx.seq_row_start.data_ptr()), ctypes.c_void_p(ctx.seq_slots.data_ptr()),
-            t, ctx.S, heads, dim, vdim, _DT[qkv.dtype], self._stream()))
+        args = (ctypes.c_void_p(qkv.data_ptr()), qkv.shape[1], q_off, k_off, v_off,
+                ctypes.c_void_p(decay.data_ptr()), ctypes.c_void_p(state.data_ptr()),
+                ctypes.c_longlong(state.stride(0)), ctypes.c_void_p(out.data_ptr()),
+                ctypes.c_void_p(ctx.seq_row_start.data_ptr()), ctypes.c_void_p(ctx.seq_slots.data_ptr()),
+                t, ctx.S, heads, dim, vdim, _DT[qkv.dtype], self._stream())
+        # bfloat16 steps that bring prompt portions: chunks of 64 rows on the matrix cores (the
+        # sums of a chunk are ordered otherwise than token by token, so the 32-bit path, whose
+        # logits do not depend on the cut to the bit, stays on the token-by-token kernel)
+        if qkv.dtype == torch.bfloat16 and ctx.max_qlen >= self.lightning_chunk_min_rows \
+                and not self.force_generic:
+            rc = self.lib.ninfer_lightning_attention_chunks(*args)
+            if rc == 0:
+                return
+            if rc < 0:
+                self._ok(rc)
+        self._ok(self.lib.ninfer_lightning_attention(*args))
 
     def _latent_args(self, ctx, pool, block_table, heads, dim, rank, rot_dim, rot_n, page_size,
                      dtype):

@@ -125,8 +125,10 @@ def test_lightning_in_portions(ops, dtype, heads, dim, vdim):
     """Two requests cut into portions of many sizes against the recurrence run whole; one
     head does not decay at all, one forgets within a few tokens."""
     torch.manual_seed(heads * 7 + dim)
-    lens = [150, 31]
+    lens = [330, 31] if dim == 64 else [150, 31]
     decay = ([1.0, 0.3, 0.9, 0.99, 0.97] * 2)[:heads]
+    if dim == 16:
+        decay = [0.0]    # a head that forgets everything at once
     qk, vw = heads * dim, heads * vdim
     rows = [(torch.randn(n, 2 * qk + vw + 11) * 1.5).to(dtype) for n in lens]
     silu = plain_getodra.silu
@@ -139,7 +141,11 @@ def test_lightning_in_portions(ops, dtype, heads, dim, vdim):
                                      decay))
     state_all = torch.zeros(4, heads * dim * vdim + 9, device=DEV)
     state = state_all[:, 9:]
+    # (bfloat16 steps whose longest portion has 8 rows or more run in chunks of 64 on the matrix
+    # cores, the others token by token: both kinds follow each other on the same state)
     steps = [[64, 0], [1, 7], [1, 1], [2, 2], [33, 1], [1, 1], [17, 16], [30, 3], [1, 0]]
+    if dim == 64:
+        steps = [[130, 0], [1, 7], [1, 1], [2, 2], [65, 1], [1, 1], [64, 16], [63, 3], [3, 0]]
     assert [sum(s[r] for s in steps) for r in range(2)] == lens
     got = [torch.zeros(n, heads, vdim, dtype=torch.float64) for n in lens]
     dec = torch.tensor(decay, device=DEV)
