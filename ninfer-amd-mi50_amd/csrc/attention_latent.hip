@@ -261,6 +261,7 @@ typedef float lat_f32x16 __attribute__((ext_vector_type(16)));
 constexpr int kLatRows = 32;      // (token, head) rows per block
 constexpr int kLatKeys = 64;      // keys per tile
 constexpr int kLatColTiles = 4;   // 32-column tiles of the output per wave: latent sizes up to 512
+constexpr int kLatPieces = 20;    // 16-byte pieces of a tile per thread: cached rows of up to 640 numbers
 
 struct LatentTilePlan {
   int tiles;        // upper bound of row tiles over all requests
@@ -275,6 +276,7 @@ struct LatentTilePlan {
 static bool latent_tile_takes(const LatentArgs& a) {
   const int Dk = a.R + a.rd;
   return a.dtype == kBF16 && !a.force_plain && Dk % 8 == 0 && a.R <= 32 * 4 * kLatColTiles &&
+         kLatKeys * (Dk / 8) <= 256 * kLatPieces &&
          (a.page_size & (a.page_size - 1)) == 0 && a.seq_row_start && a.seq_pos0 && a.S > 0 &&
          ((uintptr_t)a.pool % 16 == 0);
 }
@@ -318,11 +320,16 @@ __global__ __launch_bounds__(256) void latent_attention_tile_kernel(LatentArgs a
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int lr = lane & 31, lk = lane >> 5;
 
-  // which request and which of its row tiles is this block's?
+  // Which request and which of its row tiles is this block's? The tiles are dealt out from
+  // the last one backwards: within a request the later tiles see more keys and run longer,
+  // and the long ones should start first.
   int s = -1, lt = 0;
   {
-    int left = blockIdx.x;
-    for (int i = 0; i < a.S; ++i) {
+    int total = 0;
+    for (int i = 0; i < a.S; ++i)
+      total += ((a.seq_row_start[i + 1] - a.seq_row_start[i]) * H + kLatRows - 1) / kLatRows;
+    int left = total - 1 - (int)blockIdx.x;
+    for (int i = 0; i < a.S && left >= 0; ++i) {
       const int n = (a.seq_row_start[i + 1] - a.seq_row_start[i]) * H;
       const int nt = (n + kLatRows - 1) / kLatRows;
       if (left < nt) {
@@ -359,7 +366,10 @@ __global__ __launch_bounds__(256) void latent_attention_tile_kernel(LatentArgs a
     }
     Qs[e] = (__bf16)v;
   }
-  for (int e = tid; e < kLatKeys * pl.kstr; e += 256) Ks[e] = (__bf16)0.f;   // the pads stay zero
+  {   // the columns of a key's row beyond its numbers are read as zeros and never written again
+    const int pad = pl.kstr - Dk;
+    for (int e = tid; e < kLatKeys * pad; e += 256) Ks[(e / pad) * pl.kstr + Dk + e % pad] = (__bf16)0.f;
+  }
   __syncthreads();
 
   // softmax threads: row tid / 8, keys 8 (tid % 8) .. + 7 of a tile
@@ -382,22 +392,42 @@ __global__ __launch_bounds__(256) void latent_attention_tile_kernel(LatentArgs a
   const int ks_half = (ksteps + 1) / 2;
   const int cpr = Dk / 8;   // 16-byte pieces of a cached row
 
-  for (int kt = k_begin; kt < k_end; kt += kLatKeys) {
-    // 1. the tile's keys into LDS as they lie in their pages
-    for (int e = tid; e < kLatKeys * cpr; e += 256) {
-      const int j = e / cpr, c = e % cpr;
-      const int kp = kt + j;
+  // A tile's keys travel page -> registers -> LDS; the loads of the next tile are issued before
+  // the products of this one, so that their way from memory is hidden behind them.
+  lat_bf16x8 next[kLatPieces];
+  int piece[kLatPieces];   // key of the tile << 16 | first number of the piece; -1: none
+#pragma unroll
+  for (int i = 0; i < kLatPieces; ++i) {
+    const int e = tid + 256 * i;
+    piece[i] = e < kLatKeys * cpr ? ((e / cpr) << 16) | (8 * (e % cpr)) : -1;
+  }
+  auto fetch = [&](int kt) {
+#pragma unroll
+    for (int i = 0; i < kLatPieces; ++i) {
       lat_bf16x8 v;
 #pragma unroll
       for (int x = 0; x < 8; ++x) v[x] = (__bf16)0.f;
-      if (kp <= pos_last) {
-        const int page = bt[kp >> pl.page_shift];
-        if (page >= 0)
-          v = *(const lat_bf16x8*)(pool + ((int64_t)page * a.page_size + (kp & (a.page_size - 1))) * Dk + 8 * c);
+      if (piece[i] >= 0) {
+        const int kp = kt + (piece[i] >> 16);
+        if (kp <= pos_last) {
+          const int page = bt[kp >> pl.page_shift];
+          if (page >= 0)
+            v = *(const lat_bf16x8*)(pool + ((int64_t)page * a.page_size + (kp & (a.page_size - 1))) * Dk +
+                                     (piece[i] & 0xffff));
+        }
       }
-      *(lat_bf16x8*)(Ks + j * pl.kstr + 8 * c) = v;
+      next[i] = v;
     }
-    __syncthreads();
+  };
+  if (k_begin < k_end) fetch(k_begin);
+  for (int kt = k_begin; kt < k_end; kt += kLatKeys) {
+    // 1. the tile's keys into LDS as they lie in their pages
+#pragma unroll
+    for (int i = 0; i < kLatPieces; ++i)
+      if (piece[i] >= 0)
+        *(lat_bf16x8*)(Ks + (piece[i] >> 16) * pl.kstr + (piece[i] & 0xffff)) = next[i];
+    if (kt + kLatKeys < k_end) fetch(kt + kLatKeys);
+    lds_barrier();   // (orders LDS traffic only: the next tile's loads stay under way)
     // 2. S = Q' K^T: wave w meets keys 32 (w & 1) .. + 31 over one half of the numbers
     {
       const int n = w & 1, kh = w >> 1;
@@ -407,7 +437,18 @@ __global__ __launch_bounds__(256) void latent_attention_tile_kernel(LatentArgs a
       const int s_lo = kh ? ks_half : 0, s_hi = kh ? ksteps : ks_half;
       const __bf16* qrow = Qs + lr * pl.dkp + 8 * lk;
       const __bf16* krow = Ks + (32 * n + lr) * pl.kstr + 8 * lk;
-      for (int st = s_lo; st < s_hi; ++st) {
+      int st = s_lo;
+      for (; st + 6 <= s_hi; st += 6) {   // six steps' operands are read before the first product
+        lat_bf16x8 qf[6], kf[6];
+#pragma unroll
+        for (int u = 0; u < 6; ++u) {
+          qf[u] = *(const lat_bf16x8*)(qrow + 16 * (st + u));
+          kf[u] = *(const lat_bf16x8*)(krow + 16 * (st + u));
+        }
+#pragma unroll
+        for (int u = 0; u < 6; ++u) sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qf[u], kf[u], sacc, 0, 0, 0);
+      }
+      for (; st < s_hi; ++st) {
         const lat_bf16x8 qf = *(const lat_bf16x8*)(qrow + 16 * st);
         const lat_bf16x8 kf = *(const lat_bf16x8*)(krow + 16 * st);
         sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qf, kf, sacc, 0, 0, 0);
@@ -419,7 +460,7 @@ __global__ __launch_bounds__(256) void latent_attention_tile_kernel(LatentArgs a
 #pragma unroll
         for (int r = 0; r < 4; ++r) sp[(8 * q + 4 * lk + r) * kLatKeys] = sacc[4 * q + r];
     }
-    __syncthreads();
+    lds_barrier();   // (orders LDS traffic only: the next tile's loads stay under way)
     // 3. softmax of the tile, 32-bit: eight lanes per row
     {
       float sv[8];
@@ -459,7 +500,7 @@ __global__ __launch_bounds__(256) void latent_attention_tile_kernel(LatentArgs a
       *(lat_bf16x8*)(Ps + sm_row * (kLatKeys + 8) + 8 * sm_part) = pv;
       if (sm_part == 0) alpha_s[sm_row] = al;
     }
-    __syncthreads();
+    lds_barrier();   // (orders LDS traffic only: the next tile's loads stay under way)
     // 4. O = O alpha + P V on this wave's column tiles
     {
       const float al = alpha_s[lr];   // every register of the lane belongs to row lr
@@ -485,7 +526,7 @@ __global__ __launch_bounds__(256) void latent_attention_tile_kernel(LatentArgs a
         }
       }
     }
-    __syncthreads();
+    lds_barrier();   // (orders LDS traffic only: the next tile's loads stay under way)
   }
 
   if (sm_part == 0) {

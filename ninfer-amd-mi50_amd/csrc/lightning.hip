@@ -132,6 +132,7 @@ extern "C" int ninfer_lightning_attention(const void* qkv, int stride, int q_off
 namespace ninfer {
 
 typedef float lt_f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 lt_bf16x8 __attribute__((ext_vector_type(8)));
 constexpr int kLtChunk = 64;
 constexpr int kLtStateTiles = 4;   // 32-row tiles of the state per carrying wave: dim up to 256
 
@@ -152,6 +153,7 @@ __global__ __launch_bounds__(256) void lightning_chunk_kernel(
   float* Vs = Ks + kLtChunk * qs;         // [64][33]
   float* As = Vs + kLtChunk * 33;         // [64][65]
   float* Ss = As + kLtChunk * 65;         // [dim32][33]
+  float* Ws = Ss + ((dim + 31) / 32 * 32) * 33;   // [64] d^(L - 1 - j) of the chunk's rows
   const int s = blockIdx.x, h = blockIdx.y, c0 = 32 * blockIdx.z;
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, lr = lane & 31, lk = lane >> 5;
   const int r0 = seq_row_start[s], n = seq_row_start[s + 1] - r0;
@@ -161,6 +163,9 @@ __global__ __launch_bounds__(256) void lightning_chunk_kernel(
   const float dec = decay[h];
   const float log2d = log2f(dec);
   const bool col_ok = c0 + lr < vdim;
+  // rows of bfloat16 whose q and k parts start at multiples of 16 bytes
+  const bool wide = sizeof(T) == 2 && dim % 8 == 0 && stride % 8 == 0 && q_off % 8 == 0 &&
+                    k_off % 8 == 0 && ((uintptr_t)qkv % 16 == 0);
 
   // the state: in the accumulators of waves 2 and 3 (tiles w - 2, w, ...), a copy in LDS
   lt_f32x16 sacc[kLtStateTiles];
@@ -189,16 +194,41 @@ __global__ __launch_bounds__(256) void lightning_chunk_kernel(
   for (int i0 = 0; i0 < n; i0 += kLtChunk) {
     const int L = min(kLtChunk, n - i0);
     // 1. the chunk's q, k (all of the head's numbers) and this block's value columns
-    for (int e = tid; e < kLtChunk * dim; e += 256) {
-      const int i = e / dim, d = e % dim;
-      float qv = 0.f, kv = 0.f;
-      if (i < L) {
-        const T* row = qkv + (int64_t)(r0 + i0 + i) * stride;
-        qv = silu_f(to_f32(row[q_off + h * dim + d]));
-        kv = silu_f(to_f32(row[k_off + h * dim + d]));
+    if (wide) {   // eight neighbouring numbers per load
+      const int per_row = dim / 8;
+      for (int e = tid; e < kLtChunk * per_row; e += 256) {
+        const int i = e / per_row, d = 8 * (e % per_row);
+        float qv[8], kv[8];
+#pragma unroll
+        for (int x = 0; x < 8; ++x) qv[x] = kv[x] = 0.f;
+        if (i < L) {
+          const T* row = qkv + (int64_t)(r0 + i0 + i) * stride;
+          const lt_bf16x8 a = *(const lt_bf16x8*)(row + q_off + h * dim + d);
+          const lt_bf16x8 b = *(const lt_bf16x8*)(row + k_off + h * dim + d);
+#pragma unroll
+          for (int x = 0; x < 8; ++x) {
+            qv[x] = silu_f((float)a[x]);
+            kv[x] = silu_f((float)b[x]);
+          }
+        }
+#pragma unroll
+        for (int x = 0; x < 8; ++x) {
+          Qs[i * qs + d + x] = qv[x];
+          Ks[i * qs + d + x] = kv[x];
+        }
       }
-      Qs[i * qs + d] = qv;
-      Ks[i * qs + d] = kv;
+    } else {
+      for (int e = tid; e < kLtChunk * dim; e += 256) {
+        const int i = e / dim, d = e % dim;
+        float qv = 0.f, kv = 0.f;
+        if (i < L) {
+          const T* row = qkv + (int64_t)(r0 + i0 + i) * stride;
+          qv = silu_f(to_f32(row[q_off + h * dim + d]));
+          kv = silu_f(to_f32(row[k_off + h * dim + d]));
+        }
+        Qs[i * qs + d] = qv;
+        Ks[i * qs + d] = kv;
+      }
     }
     for (int e = tid; e < kLtChunk * 32; e += 256) {
       const int i = e >> 5, c = e & 31;
@@ -207,6 +237,7 @@ __global__ __launch_bounds__(256) void lightning_chunk_kernel(
         vv = silu_f(to_f32(qkv[(int64_t)(r0 + i0 + i) * stride + v_off + h * vdim + c0 + c]));
       Vs[i * 33 + c] = vv;
     }
+    if (tid < kLtChunk) Ws[tid] = tid < L ? decay_pow(log2d, L - 1 - tid) : 0.f;
     __syncthreads();   // (also: the state's copy in LDS is the one before this chunk)
     // 2. A[i][j] = d^(i - j) q_i . k_j for j <= i: wave w has rows 32 (w / 2).., keys 32 (w % 2)..
     {
@@ -217,7 +248,8 @@ __global__ __launch_bounds__(256) void lightning_chunk_kernel(
       if (nj <= mi) {
         const float* qrow = Qs + (32 * mi + lr) * qs + lk;
         const float* krow = Ks + (32 * nj + lr) * qs + lk;
-        for (int d = 0; d + 1 < dim + 1 && d < dim; d += 2) {
+#pragma unroll 8
+        for (int d = 0; d < dim; d += 2) {
           const float qa = (d + lk < dim) ? qrow[d] : 0.f;
           const float kb = (d + lk < dim) ? krow[d] : 0.f;
           a = __builtin_amdgcn_mfma_f32_32x32x2f32(qa, kb, a, 0, 0, 0);
@@ -240,10 +272,12 @@ __global__ __launch_bounds__(256) void lightning_chunk_kernel(
       for (int i = 0; i < 16; ++i) o[i] = 0.f;
       const int row = 32 * w + lr;
       const float* arow = As + row * 65 + lk;
+#pragma unroll 8
       for (int j = 0; j < 32 * (w + 1); j += 2)
         o = __builtin_amdgcn_mfma_f32_32x32x2f32(arow[j], Vs[(j + lk) * 33 + lr], o, 0, 0, 0);
       const float carry = decay_pow(log2d, row + 1);
       const float* qrow = Qs + row * qs + lk;
+#pragma unroll 8
       for (int d = 0; d < dim; d += 2) {
         const float qa = (d + lk < dim) ? qrow[d] * carry : 0.f;
         o = __builtin_amdgcn_mfma_f32_32x32x2f32(qa, Ss[(d + lk) * 33 + lr], o, 0, 0, 0);
@@ -266,9 +300,10 @@ __global__ __launch_bounds__(256) void lightning_chunk_kernel(
 #pragma unroll
           for (int i = 0; i < 16; ++i) sacc[x][i] *= whole;
           const int d = 32 * dt + lr;
+#pragma unroll 8
           for (int j = 0; j < kLtChunk; j += 2) {
             const int jj = j + lk;
-            const float ka = (jj < L && d < dim) ? Ks[jj * qs + d] * decay_pow(log2d, L - 1 - jj) : 0.f;
+            const float ka = (jj < L && d < dim) ? Ks[jj * qs + d] * Ws[jj] : 0.f;
             sacc[x] = __builtin_amdgcn_mfma_f32_32x32x2f32(ka, Vs[jj * 33 + lr], sacc[x], 0, 0, 0);
           }
         }
@@ -308,7 +343,7 @@ __global__ __launch_bounds__(256) void lightning_chunk_kernel(
 
 static size_t lightning_chunk_lds(int dim) {
   const int dim32 = (dim + 31) / 32 * 32;
-  return ((size_t)2 * kLtChunk * (dim + 1) + kLtChunk * 33 + kLtChunk * 65 + (size_t)dim32 * 33) * sizeof(float);
+  return ((size_t)2 * kLtChunk * (dim + 1) + kLtChunk * 33 + kLtChunk * 65 + (size_t)dim32 * 33 + kLtChunk) * sizeof(float);
 }
 
 }  // namespace ninfer
