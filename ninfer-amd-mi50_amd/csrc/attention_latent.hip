@@ -356,15 +356,16 @@ __global__ __launch_bounds__(256) void latent_attention_tile_kernel(LatentArgs a
   const int* bt = a.block_table + (int64_t)s * a.bt_stride;
   const __bf16* pool = (const __bf16*)a.pool;
 
-  // Q' of the tile's rows as bfloat16, zeros in rows and columns that are not there
-  for (int e = tid; e < kLatRows * pl.dkp; e += 256) {
-    const int i = e / pl.dkp, d = e % pl.dkp;
-    float v = 0.f;
-    if (i < rows_here && d < Dk) {
+  // Q' of the tile's rows as bfloat16, zeros in rows and columns that are not there: eight
+  // threads per row
+  {
+    const int i = tid >> 3;
+    const float* src = nullptr;
+    if (i < rows_here) {
       const int f = f0 + i;
-      v = a.q_abs[((int64_t)(row0 + f / H) * H + f % H) * Dk + d];
+      src = a.q_abs + ((int64_t)(row0 + f / H) * H + f % H) * Dk;
     }
-    Qs[e] = (__bf16)v;
+    for (int d = tid & 7; d < pl.dkp; d += 8) Qs[i * pl.dkp + d] = (__bf16)((src && d < Dk) ? src[d] : 0.f);
   }
   {   // the columns of a key's row beyond its numbers are read as zeros and never written again
     const int pad = pl.kstr - Dk;
@@ -585,16 +586,21 @@ __global__ __launch_bounds__(256) void latent_attention_tile_kernel(LatentArgs a
 
 // out[t, h] = sum_c e^(m_c - M) O_c / sum_c e^(m_c - M) l_c over the chunks that saw keys.
 __global__ void latent_attention_merge_kernel(LatentArgs a, int n_chunks) {
+  extern __shared__ float smem[];   // [n_chunks] weight of each chunk: e^(m_c - M) / L (0: saw no key)
+  __shared__ float red[16];
   const int64_t th = blockIdx.x;
   const int R = a.R;
   const float* part = a.workspace + th * n_chunks * (R + 2);
   float M = -INFINITY;
   for (int c = 0; c < n_chunks; ++c) M = fmaxf(M, part[c * (R + 2) + R]);
-  float L = 0.f;
-  for (int c = 0; c < n_chunks; ++c) {
+  float mine = 0.f;
+  for (int c = threadIdx.x; c < n_chunks; c += blockDim.x) {
     const float m = part[c * (R + 2) + R];
-    if (m > -INFINITY) L += expf(m - M) * part[c * (R + 2) + R + 1];
+    const float wgt = m > -INFINITY ? expf(m - M) : 0.f;
+    smem[c] = wgt;
+    mine += wgt * part[c * (R + 2) + R + 1];
   }
+  const float L = block_sum(mine, red);   // (its barriers publish the weights)
   float inv = L > 0.f ? 1.f / L : 0.f;
   if (a.gate) {
     const int t = (int)(th / a.Hq), h = (int)(th % a.Hq);
@@ -605,8 +611,8 @@ __global__ void latent_attention_merge_kernel(LatentArgs a, int n_chunks) {
   for (int d = threadIdx.x; d < R; d += blockDim.x) {
     float o = 0.f;
     for (int c = 0; c < n_chunks; ++c) {
-      const float m = part[c * (R + 2) + R];
-      if (m > -INFINITY) o += expf(m - M) * part[c * (R + 2) + d];
+      const float wgt = smem[c];
+      if (wgt > 0.f) o = fmaf(wgt, part[c * (R + 2) + d], o);
     }
     orow[d] = (__bf16)(o * inv);
   }
@@ -630,7 +636,7 @@ static int latent_attention_tile(const LatentArgs& a, hipStream_t stream) {
   NINFER_LAUNCH_CHECK();
   if (p.n_chunks > 1) {
     const int block = a.R >= 256 ? 256 : (a.R + 63) / 64 * 64;
-    latent_attention_merge_kernel<<<(unsigned)((int64_t)a.T * a.Hq), block, 0, stream>>>(a, p.n_chunks);
+    latent_attention_merge_kernel<<<(unsigned)((int64_t)a.T * a.Hq), block, p.n_chunks * sizeof(float), stream>>>(a, p.n_chunks);
     NINFER_LAUNCH_CHECK();
   }
   return 0;

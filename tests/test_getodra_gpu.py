@@ -512,6 +512,32 @@ def test_long_decoding(case, dtype):
         case["ref"][dtype], case["noise"][dtype] = saved
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decoding_from_a_captured_graph(case, dtype):
+    """Decode-only steps replayed from a HIP graph (the first step of a shape runs eagerly, the
+    second is captured, the rest are replays): two requests decoded side by side for dozens of
+    steps, every replay against the plain implementation."""
+    runner = make_runner(case, dtype, use_graph=True)
+    reqs = {k: case["reqs"][k] for k in ("r0", "r4")}
+    from ninfer_amd.engine import Chunk
+    slots = {k: runner.open() for k in reqs}
+    heads = {k: len(v) - 30 for k, v in reqs.items()}
+    got = {k: [] for k in reqs}
+    logits = runner.step([Chunk(slots[k], reqs[k][:heads[k]], list(range(heads[k]))) for k in reqs])
+    o = 0
+    for k in reqs:
+        got[k].append(logits[o:o + heads[k]].float().cpu())
+        o += heads[k]
+    for i in range(30):
+        logits = runner.step([Chunk(slots[k], [reqs[k][heads[k] + i]], [0]) for k in reqs])
+        for j, k in enumerate(reqs):
+            got[k].append(logits[j:j + 1].float().cpu().clone())
+    assert len(runner._graphs) >= 1
+    for k in reqs:
+        runner.close(slots[k])
+    check_logits(case, dtype, {k: torch.cat(v) for k, v in got.items()}, "graph replay")
+
+
 def test_greedy_generation_through_the_scheduler(case):
     """The framework's own entry point: prompts of unequal length generated greedily by the
     scheduler (admission, portions under a token budget, batched decoding, sampling kernel),
