@@ -278,7 +278,7 @@ static bool latent_tile_takes(const LatentArgs& a) {
   return a.dtype == kBF16 && !a.force_plain && Dk % 8 == 0 && a.R <= 32 * 4 * kLatColTiles &&
          kLatKeys * (Dk / 8) <= 256 * kLatPieces &&
          (a.page_size & (a.page_size - 1)) == 0 && a.seq_row_start && a.seq_pos0 && a.S > 0 &&
-         ((uintptr_t)a.pool % 16 == 0);
+         ((uintptr_t)a.pool % 16 == 0) && ((uintptr_t)a.q_abs % 16 == 0);
 }
 
 static LatentTilePlan latent_tile_plan(const LatentArgs& a) {
@@ -365,7 +365,18 @@ __global__ __launch_bounds__(256) void latent_attention_tile_kernel(LatentArgs a
       const int f = f0 + i;
       src = a.q_abs + ((int64_t)(row0 + f / H) * H + f % H) * Dk;
     }
-    for (int d = tid & 7; d < pl.dkp; d += 8) Qs[i * pl.dkp + d] = (__bf16)((src && d < Dk) ? src[d] : 0.f);
+    // (the row has a multiple of 8 numbers and so has its place in LDS: four at a time, and
+    // several loads under way)
+#pragma unroll 5
+    for (int d = 4 * (tid & 7); d < pl.dkp; d += 32) {
+      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (src && d < Dk) v = *(const float4*)(src + d);
+      __bf16* dst = Qs + i * pl.dkp + d;
+      dst[0] = (__bf16)v.x;
+      dst[1] = (__bf16)v.y;
+      dst[2] = (__bf16)v.z;
+      dst[3] = (__bf16)v.w;
+    }
   }
   {   // the columns of a key's row beyond its numbers are read as zeros and never written again
     const int pad = pl.kstr - Dk;
