@@ -480,7 +480,7 @@ def getodra_config(z: dict) -> dict:
     latent = {"heads": z["heads"], "dim": z["head"] - z["rot"], "rot_dim": z["rot"],
               "vdim": z["vdim"], "kv_rank": z["rank"], "scale": z["head"] ** -0.5,
               "rot": {"base": 10000.0, "dims": z["rot"],
-                      "scaling": {"factor": 4.0, "original": 1024, "fast": 32.0, "slow": 1.0}}}
+                      "scaling": {"factor": 8.0, "original": 1024, "fast": 16.0, "slow": 2.0}}}
     lightning = {"heads": z["heads"], "dim": z["head"], "vdim": z["vdim"],
                  "decay": [1.0 - 2.0 ** -(3 + 5 * h / max(z["heads"] - 1, 1)) for h in range(z["heads"])]}
     mlp = {"kind": "dense", "ff": z["ff"]}

@@ -131,7 +131,7 @@ __global__ void latent_kv_write_kernel(LatentArgs a) {
   }
 }
 
-constexpr int kLatentMaxPerLane = 8;   // latent sizes up to 512
+constexpr int kLatentMaxPerLane = 16;   // latent sizes up to 1024
 
 template <typename T>
 __global__ __launch_bounds__(64) void latent_attention_kernel(LatentArgs a) {

@@ -60,7 +60,7 @@ def test_config_errors(bad):
 
 
 @pytest.mark.parametrize("rot", [
-    {"base": 20000.0, "dims": 32, "scaling": {"factor": 4.0, "original": 1024, "fast": 32.0, "slow": 1.0}},
+    {"base": 30000.0, "dims": 32, "scaling": {"factor": 6.0, "original": 1024, "fast": 24.0, "slow": 1.5}},
     {"base": 10000.0, "dims": 8, "scaling": {"factor": 8.0, "original": 64, "fast": 16.0, "slow": 2.0}},
     {"base": 500.0, "dims": 6},
 ])

@@ -120,7 +120,7 @@ def _plain_lightning(q, k, v, decay):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("heads,dim,vdim", [(5, 12, 20), (2, 64, 32), (1, 16, 16), (3, 40, 300)])
+@pytest.mark.parametrize("heads,dim,vdim", [(5, 12, 20), (2, 64, 48), (1, 16, 16), (3, 40, 300)])
 def test_lightning_in_portions(ops, dtype, heads, dim, vdim):
     """Two requests cut into portions of many sizes against the recurrence run whole; one
     head does not decay at all, one forgets within a few tokens."""
@@ -164,7 +164,7 @@ def test_lightning_in_portions(ops, dtype, heads, dim, vdim):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("heads,k,n", [(3, 24, 40), (4, 64, 128), (1, 16, 32), (5, 40, 20)])
+@pytest.mark.parametrize("heads,k,n", [(3, 24, 40), (4, 64, 160), (1, 16, 32), (5, 40, 20), (2, 12, 10)])
 @pytest.mark.parametrize("rows", [1, 7, 70])
 def test_per_head_linear(ops, dtype, heads, k, n, rows):
     torch.manual_seed(rows + k)
@@ -536,6 +536,36 @@ def test_decoding_from_a_captured_graph(case, dtype):
     for k in reqs:
         runner.close(slots[k])
     check_logits(case, dtype, {k: torch.cat(v) for k, v in got.items()}, "graph replay")
+
+
+@pytest.mark.parametrize("kind", ["lightning", "latent_attention"])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_models_of_one_kind_of_layer(kind, dtype, tmp_path):
+    """A model with lightning layers alone holds no pages at all, one with latent attention
+    alone no lightning state; widths and sizes that are no multiple of 8."""
+    import ninfer_amd
+    from ninfer_amd import EngineOptions, load_model
+    raw = getodra_cases.config_odd()
+    raw["width"], raw["vocab"] = 52, 90
+    keep = [l for l in raw["layers"] if l["type"] == kind and "weights_of" not in l]
+    again = dict(keep[0], weights_of=0)
+    raw["layers"] = [keep[0], again]
+    if kind == "latent_attention":
+        raw["layers"][0]["mixer"].update(dim=14, rot_dim=6, kv_rank=23, vdim=9)
+        raw["layers"][0]["mixer"]["rot"]["dims"] = 6
+        raw["layers"][1] = dict(raw["layers"][0], weights_of=0)
+    d = str(tmp_path)
+    ninfer_amd.write_random_model(d, raw, 3, dtype=dtype, std=STD)
+    cfg, w = util.read_folder(d)
+    toks = util.random_tokens(45, raw["vocab"], 8)
+    ref = plain_getodra.forward(w, cfg, toks)
+    runner = load_model(d, EngineOptions(dtype=dtype, max_context=raw["max_positions"], num_sequences=2,
+                                         page_size=8, num_pages=12, check_pages=True))
+    assert bool(runner.cache.groups) == (kind == "latent_attention")
+    case = {"name": kind, "ref": {dtype: {"x": ref}}, "noise": {dtype: {"x": noise_of(cfg, w, toks, ref)}}}
+    for sched in (util.schedule_whole("x", toks), util.schedule_tail("x", toks, 20),
+                  util.schedule_portions("x", toks, seed=1)):
+        check_logits(case, dtype, util.run_schedule(runner, sched), "one kind of layer")
 
 
 def test_greedy_generation_through_the_scheduler(case):
