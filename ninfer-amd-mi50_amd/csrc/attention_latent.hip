@@ -52,6 +52,7 @@ struct LatentArgs {
   long long workspace_floats;
   int S;
   int max_kv_len;           // host-side bound that sizes the chunks
+  int max_qlen;             // host-side: the most rows a request brings (1: a decode-only step)
   int force_plain;          // tests: the plain kernel whatever the shape
   int dkv_stride;
   int gate_stride;
@@ -288,9 +289,14 @@ static LatentTilePlan latent_tile_plan(const LatentArgs& a) {
   const int cols = (a.R + 31) / 32 * 32;
   p.dkp = dk16 + 8;
   p.kstr = (dk16 > cols ? dk16 : cols) + 8;
-  p.tiles = (int)(((int64_t)a.T * a.Hq + kLatRows - 1) / kLatRows) + a.S;
+  // row tiles: in a decode-only step every request has the same number; otherwise a bound
+  // (a request's last tile may be partial; tiles that do not exist exit at once)
+  p.tiles = a.max_qlen == 1 ? a.S * ((a.Hq + kLatRows - 1) / kLatRows)
+                            : (int)(((int64_t)a.T * a.Hq + kLatRows - 1) / kLatRows) + a.S;
   const int key_tiles = (a.max_kv_len + kLatKeys - 1) / kLatKeys;
-  int want = (2 * device_cu_count() + p.tiles - 1) / p.tiles;   // blocks enough for two a CU
+  // a block fills a CU (its LDS and registers): one block per CU, each with as long a walk as
+  // that allows, since a block's start (Q', its first tile) costs as much as two tiles
+  int want = device_cu_count() / p.tiles;
   if (want > key_tiles) want = key_tiles;
   if (want < 1) want = 1;
   const int tiles_per_chunk = (key_tiles + want - 1) / want;
@@ -603,6 +609,7 @@ __global__ void latent_attention_merge_kernel(LatentArgs a, int n_chunks) {
   const int R = a.R;
   const float* part = a.workspace + th * n_chunks * (R + 2);
   float M = -INFINITY;
+#pragma unroll 8
   for (int c = 0; c < n_chunks; ++c) M = fmaxf(M, part[c * (R + 2) + R]);
   float mine = 0.f;
   for (int c = threadIdx.x; c < n_chunks; c += blockDim.x) {
@@ -620,11 +627,11 @@ __global__ void latent_attention_merge_kernel(LatentArgs a, int n_chunks) {
   }
   __bf16* orow = (__bf16*)a.out + th * R;
   for (int d = threadIdx.x; d < R; d += blockDim.x) {
+    // (a chunk that saw no key left zeros and has weight 0: no branch, so that the loads of
+    // several chunks are under way together)
     float o = 0.f;
-    for (int c = 0; c < n_chunks; ++c) {
-      const float wgt = smem[c];
-      if (wgt > 0.f) o = fmaf(wgt, part[c * (R + 2) + d], o);
-    }
+#pragma unroll 8
+    for (int c = 0; c < n_chunks; ++c) o = fmaf(smem[c], part[c * (R + 2) + d], o);
     orow[d] = (__bf16)(o * inv);
   }
 }

@@ -96,7 +96,8 @@ class _LatentArgs(ctypes.Structure):
                 ("row_seq", ctypes.c_void_p), ("seq_row_start", ctypes.c_void_p),
                 ("seq_pos0", ctypes.c_void_p), ("workspace", ctypes.c_void_p),
                 ("workspace_floats", ctypes.c_longlong), ("S", ctypes.c_int),
-                ("max_kv_len", ctypes.c_int), ("force_plain", ctypes.c_int),
+                ("max_kv_len", ctypes.c_int), ("max_qlen", ctypes.c_int),
+                ("force_plain", ctypes.c_int),
                 ("dkv_stride", ctypes.c_int),
                 ("gate_stride", ctypes.c_int), ("bt_stride", ctypes.c_int), ("T", ctypes.c_int),
                 ("Hq", ctypes.c_int), ("dim", ctypes.c_int), ("R", ctypes.c_int),
@@ -968,7 +969,8 @@ class HipOps:
         a.pool, a.block_table = pool.data_ptr(), block_table.data_ptr()
         a.positions, a.row_seq = ctx.positions.data_ptr(), ctx.row_seq.data_ptr()
         a.seq_row_start, a.seq_pos0 = ctx.seq_row_start.data_ptr(), ctx.seq_pos0.data_ptr()
-        a.S, a.max_kv_len, a.force_plain = ctx.S, ctx.max_kv_len, 1 if self.force_generic else 0
+        a.S, a.max_kv_len, a.max_qlen = ctx.S, ctx.max_kv_len, ctx.max_qlen
+        a.force_plain = 1 if self.force_generic else 0
         a.bt_stride, a.T, a.Hq, a.dim, a.R, a.rd, a.rot_n = \
             block_table.shape[1], ctx.T, heads, dim, rank, rot_dim, rot_n
         a.page_size, a.dtype = page_size, _DT[dtype]
