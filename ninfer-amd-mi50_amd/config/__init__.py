@@ -2,6 +2,7 @@ from .base import ConfigError, KeyReader, architecture_name, read_config_json
 from .getodra import GetodraConfig
 from .options import EngineOptions
 from .qwen2_moe import Qwen2MoeConfig
+from .sosepel import SosepelConfig
 
 __all__ = ["ConfigError", "KeyReader", "architecture_name", "read_config_json",
-           "EngineOptions", "GetodraConfig", "Qwen2MoeConfig"]
+           "EngineOptions", "GetodraConfig", "Qwen2MoeConfig", "SosepelConfig"]

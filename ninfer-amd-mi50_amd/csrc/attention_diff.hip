@@ -1,0 +1,274 @@
+// Differential attention over the paged cache (see attention_diff.h for what it computes):
+// the write of keys and values into pages, the plain kernel (one wave per row and query
+// head, both maps at once; the 32-bit path, sizes the matrix-core kernel refuses, and single
+// rows with their contexts cut into chunks), and the merge of such chunks.
+//
+// Keys are walked in tiles of 64 aligned to absolute positions with an online softmax per
+// map, so without chunks the order of every sum depends on the row's own position only.
+// Scores, both softmaxes, the difference and the head's norm are 32-bit.
+#include "attention_diff.h"
+
+namespace ninfer {
+
+constexpr int kMaxVPerLane = 8;   // value sizes up to 512
+
+// temp(p) = 1 + coef ln(floor((p + 1) / every) + 1)
+__device__ __forceinline__ float query_temperature(int pos, float coef, int every) {
+  if (coef == 0.f) return 1.f;
+  return 1.f + coef * logf((float)((pos + 1) / every) + 1.f);
+}
+
+// k and v of every row into the request's pages.
+template <typename T>
+__global__ void diff_kv_write_kernel(DiffAttnArgs a) {
+  const int t = blockIdx.x;
+  const int pos = a.positions[t];
+  const int page = a.block_table[(int64_t)a.row_seq[t] * a.bt_stride + pos / a.page_size];
+  const int slot = pos % a.page_size;
+  const int kd = 2 * a.dim;
+  const T* row = (const T*)a.qkv + (int64_t)t * a.q_stride + a.Hq * kd;
+  T* kp = (T*)a.kpool;
+  T* vp = (T*)a.vpool;
+  const int nk = a.Hkv * kd, nv = a.Hkv * a.vdim;
+  for (int i = threadIdx.x; i < nk; i += blockDim.x) {
+    const int g = i / kd, d = i % kd;
+    kp[(((int64_t)page * a.Hkv + g) * a.page_size + slot) * kd + d] = row[i];
+  }
+  for (int i = threadIdx.x; i < nv; i += blockDim.x) {
+    const int g = i / a.vdim, d = i % a.vdim;
+    vp[(((int64_t)page * a.Hkv + g) * a.page_size + slot) * a.vdim + d] = row[nk + i];
+  }
+}
+
+// o = a1 / l1 - lambda a2 / l2 over the lane's value columns, the head's norm, the store.
+template <typename T>
+__device__ __forceinline__ void diff_finish(const DiffAttnArgs& a, const float* acc1,
+                                            const float* acc2, float l1, float l2, T* orow,
+                                            int lane) {
+  const float i1 = 1.f / l1, i2 = a.lambda / l2;
+  float o[kMaxVPerLane];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < kMaxVPerLane; ++i) {
+    const int d = lane + i * 64;
+    o[i] = d < a.vdim ? acc1[i] * i1 - acc2[i] * i2 : 0.f;
+    ss += o[i] * o[i];
+  }
+  float r = a.out_scale;
+  if (a.eps >= 0.f) r *= 1.f / sqrtf(wave_sum(ss) / (float)a.vdim + a.eps);
+#pragma unroll
+  for (int i = 0; i < kMaxVPerLane; ++i) {
+    const int d = lane + i * 64;
+    if (d < a.vdim) orow[d] = from_f32<T>(o[i] * r);
+  }
+}
+
+// One wave per (row, query head, chunk of the context). n_chunks == 1: the whole context,
+// result written to out; else keys [c chunk, (c + 1) chunk) and partial results
+// {m1, l1, m2, l2, acc1[vdim], acc2[vdim]} into the workspace.
+template <typename T>
+__global__ __launch_bounds__(64) void diff_attention_plain_kernel(DiffAttnArgs a, int chunk,
+                                                                  int n_chunks) {
+  extern __shared__ float smem[];
+  const int kd = 2 * a.dim;
+  float* q_s = smem;                  // [2 dim]
+  float* p1_s = q_s + kd;             // [64]
+  float* p2_s = p1_s + 64;            // [64]
+  int64_t* off_s = (int64_t*)(p2_s + 64 + ((kd & 1) ? 1 : 0));   // [64] element offset of each value row
+
+  const int t = blockIdx.x, h = blockIdx.y, c = blockIdx.z, lane = threadIdx.x;
+  const int g = h / (a.Hq / a.Hkv);
+  const int pos = a.positions[t];
+  const int* bt = a.block_table + (int64_t)a.row_seq[t] * a.bt_stride;
+  const int first = n_chunks > 1 ? c * chunk : 0;
+  const int last = n_chunks > 1 ? min(pos, first + chunk - 1) : pos;
+  const float qscale = a.scale * query_temperature(pos, a.t_coef, a.t_every);
+  const T* kpool = (const T*)a.kpool;
+  const T* vpool = (const T*)a.vpool;
+
+  const T* qr = (const T*)a.qkv + (int64_t)t * a.q_stride + h * kd;
+  for (int d = lane; d < kd; d += 64) q_s[d] = to_f32(qr[d]);
+  __syncthreads();
+
+  float m1 = -INFINITY, l1 = 0.f, m2 = -INFINITY, l2 = 0.f;
+  float acc1[kMaxVPerLane], acc2[kMaxVPerLane];
+#pragma unroll
+  for (int i = 0; i < kMaxVPerLane; ++i) acc1[i] = acc2[i] = 0.f;
+
+  for (int tile = first; tile <= last; tile += 64) {   // chunks are multiples of 64
+    const int j = tile + lane;
+    const bool valid = j <= last;
+    float s1 = -INFINITY, s2 = -INFINITY;
+    int64_t voff = 0;
+    if (valid) {
+      const int page = bt[j / a.page_size];
+      const int64_t at = ((int64_t)page * a.Hkv + g) * a.page_size + (j % a.page_size);
+      voff = at * a.vdim;
+      const T* kr = kpool + at * kd;
+      float d1 = 0.f, d2 = 0.f;
+      for (int d = 0; d < a.dim; ++d) d1 = fmaf(q_s[d], to_f32(kr[d]), d1);
+      for (int d = 0; d < a.dim; ++d) d2 = fmaf(q_s[a.dim + d], to_f32(kr[a.dim + d]), d2);
+      s1 = d1 * qscale;
+      s2 = d2 * qscale;
+      if (a.cap > 0.f) {
+        s1 = a.cap * tanhf(s1 / a.cap);
+        s2 = a.cap * tanhf(s2 / a.cap);
+      }
+    }
+    const float n1 = fmaxf(m1, wave_max(s1)), n2 = fmaxf(m2, wave_max(s2));
+    const float p1 = valid ? expf(s1 - n1) : 0.f, p2 = valid ? expf(s2 - n2) : 0.f;
+    const float al1 = expf(m1 - n1), al2 = expf(m2 - n2);   // 0 on the first tile
+    l1 = l1 * al1 + wave_sum(p1);
+    l2 = l2 * al2 + wave_sum(p2);
+    m1 = n1;
+    m2 = n2;
+    p1_s[lane] = p1;
+    p2_s[lane] = p2;
+    off_s[lane] = voff;
+    __syncthreads();
+    const int n_keys = min(64, last - tile + 1);
+#pragma unroll
+    for (int i = 0; i < kMaxVPerLane; ++i) {
+      const int d = lane + i * 64;
+      if (d < a.vdim) {
+        float x1 = acc1[i] * al1, x2 = acc2[i] * al2;
+        for (int jj = 0; jj < n_keys; ++jj) {
+          const float v = to_f32(vpool[off_s[jj] + d]);
+          x1 = fmaf(p1_s[jj], v, x1);
+          x2 = fmaf(p2_s[jj], v, x2);
+        }
+        acc1[i] = x1;
+        acc2[i] = x2;
+      }
+    }
+    __syncthreads();
+  }
+  if (n_chunks == 1) {
+    diff_finish<T>(a, acc1, acc2, l1, l2, (T*)a.out + ((int64_t)t * a.Hq + h) * a.vdim, lane);
+    return;
+  }
+  float* part = a.workspace + (((int64_t)t * a.Hq + h) * n_chunks + c) * (4 + 2 * a.vdim);
+  if (lane == 0) {
+    part[0] = m1;
+    part[1] = l1;
+    part[2] = m2;
+    part[3] = l2;
+  }
+#pragma unroll
+  for (int i = 0; i < kMaxVPerLane; ++i) {
+    const int d = lane + i * 64;
+    if (d < a.vdim) {
+      part[4 + d] = acc1[i];
+      part[4 + a.vdim + d] = acc2[i];
+    }
+  }
+}
+
+// The chunks of a row and head put together, in the chunks' order (a chunk that starts
+// beyond the row's position holds l = 0 and counts for nothing).
+template <typename T>
+__global__ __launch_bounds__(64) void diff_attention_merge_kernel(DiffAttnArgs a, int n_chunks) {
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int stride = 4 + 2 * a.vdim;
+  const float* part = a.workspace + ((int64_t)t * a.Hq + h) * n_chunks * stride;
+  float m1 = -INFINITY, m2 = -INFINITY;
+  for (int c = 0; c < n_chunks; ++c) {
+    if (part[c * stride + 1] > 0.f) m1 = fmaxf(m1, part[c * stride]);
+    if (part[c * stride + 3] > 0.f) m2 = fmaxf(m2, part[c * stride + 2]);
+  }
+  float l1 = 0.f, l2 = 0.f;
+  float acc1[kMaxVPerLane], acc2[kMaxVPerLane];
+#pragma unroll
+  for (int i = 0; i < kMaxVPerLane; ++i) acc1[i] = acc2[i] = 0.f;
+  for (int c = 0; c < n_chunks; ++c) {
+    const float* p = part + c * stride;
+    const float w1 = p[1] > 0.f ? expf(p[0] - m1) : 0.f, w2 = p[3] > 0.f ? expf(p[2] - m2) : 0.f;
+    l1 += w1 * p[1];
+    l2 += w2 * p[3];
+#pragma unroll
+    for (int i = 0; i < kMaxVPerLane; ++i) {
+      const int d = lane + i * 64;
+      if (d < a.vdim) {
+        if (w1 > 0.f) acc1[i] = fmaf(w1, p[4 + d], acc1[i]);
+        if (w2 > 0.f) acc2[i] = fmaf(w2, p[4 + a.vdim + d], acc2[i]);
+      }
+    }
+  }
+  diff_finish<T>(a, acc1, acc2, l1, l2, (T*)a.out + ((int64_t)t * a.Hq + h) * a.vdim, lane);
+}
+
+int diff_attention_plain(const DiffAttnArgs& a, int chunk, int n_chunks, hipStream_t stream) {
+  const size_t lds = (2 * a.dim + 128 + 2) * sizeof(float) + 64 * sizeof(int64_t);
+  dim3 grid(a.T, a.Hq, n_chunks);
+  if (a.dtype == kF32) {
+    diff_attention_plain_kernel<float><<<grid, 64, lds, stream>>>(a, chunk, n_chunks);
+    if (n_chunks > 1) diff_attention_merge_kernel<float><<<dim3(a.T, a.Hq), 64, 0, stream>>>(a, n_chunks);
+  } else {
+    diff_attention_plain_kernel<bf16><<<grid, 64, lds, stream>>>(a, chunk, n_chunks);
+    if (n_chunks > 1) diff_attention_merge_kernel<bf16><<<dim3(a.T, a.Hq), 64, 0, stream>>>(a, n_chunks);
+  }
+  NINFER_LAUNCH_CHECK();
+  return 0;
+}
+
+// Single rows (a decode step): how the contexts are cut so that the launch fills the GPU.
+static void diff_chunks(const DiffAttnArgs& a, int* chunk, int* n_chunks) {
+  *chunk = 0;
+  *n_chunks = 1;
+  if (a.dtype != kBF16 || a.max_qlen != 1 || a.force_plain) return;
+  const int waves = a.T * a.Hq;
+  const int want = (8 * device_cu_count() + waves - 1) / waves;   // eight waves a CU
+  int per = (a.max_kv_len + want - 1) / want;
+  per = ((per < 256 ? 256 : per) + 63) / 64 * 64;
+  const int n = (a.max_kv_len + per - 1) / per;
+  if (n > 1) {
+    *chunk = per;
+    *n_chunks = n;
+  }
+}
+
+static int diff_check(const DiffAttnArgs& a, const char* who) {
+  NINFER_REQUIRE(a.T > 0 && a.S > 0 && a.Hq > 0 && a.Hkv > 0 && a.dim > 0 && a.vdim > 0 && a.page_size > 0,
+                 "%s: sizes must be positive", who);
+  NINFER_REQUIRE(a.Hq % a.Hkv == 0, "%s: %d query heads do not split over %d kv heads", who, a.Hq, a.Hkv);
+  NINFER_REQUIRE(a.dtype == kF32 || a.dtype == kBF16, "%s: unknown dtype %d", who, a.dtype);
+  NINFER_REQUIRE(a.vdim <= 64 * kMaxVPerLane, "%s: value size %d exceeds %d", who, a.vdim, 64 * kMaxVPerLane);
+  NINFER_REQUIRE(a.q_stride >= (a.Hq + a.Hkv) * 2 * a.dim + a.Hkv * a.vdim, "%s: rows of %d numbers are too short",
+                 who, a.q_stride);
+  NINFER_REQUIRE(a.t_coef == 0.f || a.t_every > 0, "%s: the temperature's step must be positive", who);
+  NINFER_REQUIRE(a.cap >= 0.f && a.scale > 0.f, "%s: the cap must not be negative, the scale positive", who);
+  return 0;
+}
+
+}  // namespace ninfer
+
+using namespace ninfer;
+
+extern "C" int ninfer_diff_kv_write(const DiffAttnArgs* a, hipStream_t stream) {
+  int rc = diff_check(*a, "diff_kv_write");
+  if (rc) return rc;
+  if (a->dtype == kF32) diff_kv_write_kernel<float><<<a->T, 256, 0, stream>>>(*a);
+  else diff_kv_write_kernel<bf16><<<a->T, 256, 0, stream>>>(*a);
+  NINFER_LAUNCH_CHECK();
+  return 0;
+}
+
+extern "C" long long ninfer_diff_attention_workspace_floats(const DiffAttnArgs* a) {
+  int chunk, n;
+  diff_chunks(*a, &chunk, &n);
+  return n > 1 ? (long long)a->T * a->Hq * n * (4 + 2 * a->vdim) : 0;
+}
+
+extern "C" int ninfer_diff_attention(const DiffAttnArgs* a, hipStream_t stream) {
+  int rc = diff_check(*a, "diff_attention");
+  if (rc) return rc;
+  NINFER_REQUIRE(a->out && a->qkv && a->kpool && a->vpool, "diff_attention: null tensors");
+  if (a->max_qlen > 1 && !a->force_plain && diff_attention_tiles_takes(*a))
+    return diff_attention_tiles(*a, stream);
+  int chunk, n;
+  diff_chunks(*a, &chunk, &n);
+  if (n > 1)
+    NINFER_REQUIRE(a->workspace && a->workspace_floats >= (int64_t)a->T * a->Hq * n * (4 + 2 * a->vdim),
+                   "diff_attention: the workspace is too small for %d chunks", n);
+  return diff_attention_plain(*a, chunk, n, stream);
+}

@@ -13,11 +13,12 @@ enum RouteScore : int { kScoreSoftmax = 0, kScoreSigmoid = 1 };
 // What a router computes from its logits, and where routing writes (all on the device).
 //   s_e = softmax(logits)_e, or sigmoid(logits_e)            (`score`)
 //   candidates = all experts, or with `n_group` > 1 those of the `topk_group` groups (of E /
-//            n_group neighbouring experts each) whose largest s_e + choice_bias_e is largest,
+//            n_group neighbouring experts each) whose largest s_e + choice_bias_e is largest
+//            (`group_top` > 1: whose sum of the group_top largest s_e + choice_bias_e is),
 //            ties to the lower group
 //   chosen = the k candidates with the largest s_e + choice_bias_e, ties to the lower index
-//   w_e    = s_e of the chosen (the bias decides the choice only), divided by their sum when
-//            `renorm`, times `scale`
+//   w_e    = s_e of the chosen (the bias decides the choice only), divided by their sum
+//            (+ `renorm_eps`) when `renorm`, times `scale`
 // Softmax without bias, scale 1: the reference's router (src/ops/moe.hip:65-82), which
 // always renormalises.
 struct RouteArgs {
@@ -38,6 +39,8 @@ struct RouteArgs {
   float scale;       // factor on every weight
   int n_group;       // groups of experts for a group-limited choice (0 or 1: none; at most 64)
   int topk_group;    // groups whose experts are candidates
+  int group_top;     // a group's score is the sum of its group_top largest (0 or 1: its largest)
+  float renorm_eps;  // added to the sum of the chosen scores before the division
 };
 
 // A group-limited choice asks: groups of equal size, at most 64 of them, and enough candidates
@@ -45,7 +48,8 @@ struct RouteArgs {
 inline bool route_groups_ok(const RouteArgs& rt) {
   if (rt.n_group <= 1) return rt.n_group >= 0;
   return rt.n_group <= 64 && rt.E % rt.n_group == 0 && rt.topk_group >= 1 &&
-         rt.topk_group <= rt.n_group && (long)rt.topk_group * (rt.E / rt.n_group) >= rt.k;
+         rt.topk_group <= rt.n_group && (long)rt.topk_group * (rt.E / rt.n_group) >= rt.k &&
+         rt.group_top >= 0 && rt.group_top <= rt.E / rt.n_group;
 }
 
 constexpr int kMaxExpertsPerLane = 16;  // up to 1024 experts
@@ -106,7 +110,64 @@ __device__ __forceinline__ int route_row(const float* __restrict__ row, const Ro
   bad = __any(bad);
 #pragma unroll
   for (int i = 0; i < NPL; ++i) sel[i] = lane + i * 64 < E ? (bad ? 0.f : sel[i]) : -INFINITY;
-  if (rt.n_group > 1 && rt.topk_group < rt.n_group) {
+  if (rt.n_group > 1 && rt.topk_group < rt.n_group && rt.group_top > 1) {
+    // a group's score: the sum of its group_top largest, kept by lane g for group g
+    const int per_group = E / rt.n_group;
+    float tmp[NPL];
+#pragma unroll
+    for (int i = 0; i < NPL; ++i) tmp[i] = sel[i];
+    float gscore = -INFINITY;
+    for (int g = 0; g < rt.n_group; ++g) {
+      float sum = 0.f;
+      for (int j = 0; j < rt.group_top; ++j) {
+        float best = -INFINITY;
+        int best_e = 0x7fffffff;
+#pragma unroll
+        for (int i = 0; i < NPL; ++i) {
+          const int e = lane + i * 64;
+          if (e < E && e / per_group == g && tmp[i] > best) {
+            best = tmp[i];
+            best_e = e;
+          }
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+          const float ob = __shfl_xor(best, off, 64);
+          const int oe = __shfl_xor(best_e, off, 64);
+          if (ob > best || (ob == best && oe < best_e)) {
+            best = ob;
+            best_e = oe;
+          }
+        }
+#pragma unroll
+        for (int i = 0; i < NPL; ++i)
+          if (lane + i * 64 == best_e) tmp[i] = -INFINITY;
+        sum += best;
+      }
+      if (lane == g) gscore = sum;
+    }
+    unsigned long long open_groups = 0;
+    for (int j = 0; j < rt.topk_group; ++j) {
+      float best = gscore;
+      int best_g = lane < rt.n_group ? lane : 0x7fffffff;
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) {
+        const float ob = __shfl_xor(best, off, 64);
+        const int og = __shfl_xor(best_g, off, 64);
+        if (ob > best || (ob == best && og < best_g)) {
+          best = ob;
+          best_g = og;
+        }
+      }
+      open_groups |= 1ull << best_g;
+      if (lane == best_g) gscore = -INFINITY;
+    }
+#pragma unroll
+    for (int i = 0; i < NPL; ++i) {
+      const int e = lane + i * 64;
+      if (e < E && !((open_groups >> (e / per_group)) & 1ull)) sel[i] = -INFINITY;
+    }
+  } else if (rt.n_group > 1 && rt.topk_group < rt.n_group) {
     // the groups that may be chosen from: topk_group times the group of the best remaining score
     const int per_group = E / rt.n_group;
     unsigned long long open_groups = 0;
@@ -176,7 +237,7 @@ __device__ __forceinline__ int route_row(const float* __restrict__ row, const Ro
   }
   if (lane < k) {
     ids[lane] = my_id;
-    wts[lane] = bad ? __builtin_nanf("") : (rt.renorm ? my_w / chosen_sum : my_w) * rt.scale;
+    wts[lane] = bad ? __builtin_nanf("") : (rt.renorm ? my_w / (chosen_sum + rt.renorm_eps) : my_w) * rt.scale;
   }
   return my_id;
 }

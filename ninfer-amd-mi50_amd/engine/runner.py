@@ -63,7 +63,9 @@ class ModelRunner:
         # one cache instance per plan entry that writes keys and values
         needs = []
         self._state_range: List[Optional[slice]] = []
-        floats = 0
+        # the embedding's per-request state (a previous token, where it hashes pairs) first
+        floats = getattr(spec.embedding, "state_floats", lambda: 0)()
+        self._embedding_state = slice(0, floats) if floats else None
         for call in spec.plan:
             mixer = spec.blocks[call.layer].mixer
             needs.append(mixer.cache_need() if call.cache_from is None else None)
@@ -88,6 +90,7 @@ class ModelRunner:
         self.graphs_dropped = 0
         self._holds_graphs = False
         self.graph_context_step = 1024   # a graph serves contexts up to the next multiple
+        self.tap = None   # tests: called as tap(plan entry, residual, pending) after every layer run
 
     # ---- read-back -------------------------------------------------------------
     def tensor_names(self) -> List[str]:
@@ -275,8 +278,9 @@ class ModelRunner:
             seq_row_start=views[4], seq_qlen=views[5], seq_pos0=views[6],
             max_qlen=shape["max_qlen"], max_kv_len=shape["max_kv_len"],
             all_decode=shape["max_qlen"] == 1, single_rows=shape["single_rows"])
+        es = self.cache.state[:, self._embedding_state] if self._embedding_state is not None else None
         return self.spec.forward(ctx, self._call_infos(d_tables),
-                                 views[7] if shape["wants"] else None)
+                                 views[7] if shape["wants"] else None, es, self.tap)
 
     def _step_graph(self, host: torch.Tensor, shape: dict) -> torch.Tensor:
         """Decode-only steps replayed from a captured HIP graph: one graph per

@@ -48,7 +48,8 @@ class _RouteArgs(ctypes.Structure):
                 ("choice_bias", ctypes.c_void_p), ("parts", ctypes.c_void_p),
                 ("E", ctypes.c_int), ("k", ctypes.c_int), ("renorm", ctypes.c_int),
                 ("score", ctypes.c_int), ("scale", ctypes.c_float), ("n_group", ctypes.c_int),
-                ("topk_group", ctypes.c_int)]
+                ("topk_group", ctypes.c_int), ("group_top", ctypes.c_int),
+                ("renorm_eps", ctypes.c_float)]
 
 
 BIG_TILE_ROWS = 256   # rows of a tall tile of the grouped products (the library's kGroupedTileRows)
@@ -104,6 +105,21 @@ class _LatentArgs(ctypes.Structure):
                 ("rd", ctypes.c_int), ("rot_n", ctypes.c_int), ("page_size", ctypes.c_int),
                 ("window", ctypes.c_int), ("write_kv", ctypes.c_int), ("dtype", ctypes.c_int),
                 ("eps", ctypes.c_float), ("magnitude", ctypes.c_float), ("scale", ctypes.c_float)]
+
+
+class _DiffAttnArgs(ctypes.Structure):
+    _fields_ = [("qkv", ctypes.c_void_p), ("kpool", ctypes.c_void_p), ("vpool", ctypes.c_void_p),
+                ("out", ctypes.c_void_p), ("block_table", ctypes.c_void_p),
+                ("positions", ctypes.c_void_p), ("row_seq", ctypes.c_void_p),
+                ("seq_row_start", ctypes.c_void_p), ("workspace", ctypes.c_void_p),
+                ("workspace_floats", ctypes.c_int64), ("q_stride", ctypes.c_int),
+                ("bt_stride", ctypes.c_int), ("T", ctypes.c_int), ("S", ctypes.c_int),
+                ("Hq", ctypes.c_int), ("Hkv", ctypes.c_int), ("dim", ctypes.c_int),
+                ("vdim", ctypes.c_int), ("page_size", ctypes.c_int), ("dtype", ctypes.c_int),
+                ("max_qlen", ctypes.c_int), ("max_kv_len", ctypes.c_int),
+                ("force_plain", ctypes.c_int), ("scale", ctypes.c_float), ("cap", ctypes.c_float),
+                ("t_coef", ctypes.c_float), ("t_every", ctypes.c_int), ("lam", ctypes.c_float),
+                ("eps", ctypes.c_float), ("out_scale", ctypes.c_float)]
 
 
 def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
@@ -209,6 +225,7 @@ class HipOps:
         self.lib.ninfer_stream_after.argtypes = [ctypes.c_void_p] * 3
         self.lib.ninfer_sample_few_places.restype = ctypes.c_longlong
         self.lib.ninfer_latent_attention_workspace_floats.restype = ctypes.c_longlong
+        self.lib.ninfer_diff_attention_workspace_floats.restype = ctypes.c_longlong
         self.force_generic = False  # tests: run the plain kernels whatever the shape
         self._device_index = None   # the one GPU's index, asked for at the first launch
         self._held = None           # products held back inside `together()`
@@ -611,8 +628,14 @@ class HipOps:
         if route is not None:
             self._route_now(*route[2])
 
-    def linear(self, x, w, out, bias=None):
-        """out = x w^T (+ bias); out may be 32-bit whatever the inputs are."""
+    def linear(self, x, w, out, bias=None, act=None):
+        """out = x w^T (+ bias); out may be 32-bit whatever the inputs are. `act` 'relu2': the
+        square of relu on every element of out."""
+        if act is not None:
+            _need(act == "relu2", f"linear: activation {act!r} is not 'relu2'")
+            self.linear(x, w, out, bias)
+            self.relu_square(out)
+            return
         _dev(x, "x", dims=2)
         _dev(w, "w", x.dtype, 2)
         _dev(out, "out", dims=2)
@@ -699,13 +722,16 @@ class HipOps:
 
     # ---- routing ------------------------------------------------------------------
     def _route_args(self, experts, top_k, renorm, ids, wts, r=None, score="softmax",
-                    choice_bias=None, scale=1.0, n_group=0, topk_group=0):
+                    choice_bias=None, scale=1.0, n_group=0, topk_group=0, group_top=1,
+                    renorm_eps=0.0):
         """The router's parameters and the places routing writes, as the library takes them.
         `score`: 'softmax' over all experts or 'sigmoid' of each logit; `choice_bias` [experts]
         is added to the scores for the choice of experts only (the weights are the scores);
         `scale` multiplies every weight, after the renormalisation if there is one; with
         `n_group` > 1 only the experts of the `topk_group` groups (of experts / n_group
-        neighbours each) with the largest best score (+ bias) are candidates."""
+        neighbours each) with the largest best score (+ bias) are candidates (`group_top` > 1:
+        with the largest sum of their group_top best); `renorm_eps` is added to the sum the
+        chosen scores are divided by."""
         _need(score in _SCORES, f"routing: score {score!r} is not one of {sorted(_SCORES)}")
         _need(1 <= top_k <= experts, f"routing: top_k {top_k} not in [1, {experts}]")
         if choice_bias is not None:
@@ -724,18 +750,20 @@ class HipOps:
                 parts = r.parts.data_ptr()
         args = _RouteArgs(ids.data_ptr(), wts.data_ptr(), offsets, order, t16, t64, tc,
                           _ptr(choice_bias), parts, experts, top_k, 1 if renorm else 0,
-                          _SCORES[score], float(scale), int(n_group), int(topk_group))
+                          _SCORES[score], float(scale), int(n_group), int(topk_group),
+                          int(group_top), float(renorm_eps))
         return args
 
     def router_topk(self, logits, experts, top_k, renorm, ids, wts, score="softmax",
-                    choice_bias=None, scale=1.0, n_group=0, topk_group=0):
+                    choice_bias=None, scale=1.0, n_group=0, topk_group=0, group_top=1,
+                    renorm_eps=0.0):
         _dev(logits, "logits", torch.float32, 2)
         _dev(ids, "ids", torch.int32, 2)
         _dev(wts, "wts", torch.float32, 2)
         t = logits.shape[0]
         _need(ids.shape == (t, top_k) and wts.shape == (t, top_k), "router_topk: output shapes")
         args = self._route_args(experts, top_k, renorm, ids, wts, None, score, choice_bias, scale,
-                                n_group, topk_group)
+                                n_group, topk_group, group_top, renorm_eps)
         self._ok(self.lib.ninfer_router_topk(
             ctypes.c_void_p(logits.data_ptr()), logits.shape[1], t, ctypes.byref(args),
             self._stream()))
@@ -764,7 +792,7 @@ class HipOps:
             ctypes.c_void_p(t16), ctypes.c_void_p(t64), ctypes.c_void_p(tc), self._stream()))
 
     def moe_route(self, logits, experts, top_k, renorm, r, score="softmax", choice_bias=None,
-                  scale=1.0, n_group=0, topk_group=0):
+                  scale=1.0, n_group=0, topk_group=0, group_top=1, renorm_eps=0.0):
         """Scores + top-k per row (see `_route_args` for the router's parameters) and the
         grouping by expert, into the routing record `r` (ids, weights, offsets, order, tile
         lists): one launch for up to 16 rows (one block does both), two for more (top-k by
@@ -782,7 +810,7 @@ class HipOps:
               and r.offsets.shape[0] == experts + 1 and r.order.shape[0] == t * top_k,
               "moe_route: output sizes")
         rargs = self._route_args(experts, top_k, renorm, r.ids, r.weights, r, score, choice_bias,
-                                 scale, n_group, topk_group)
+                                 scale, n_group, topk_group, group_top, renorm_eps)
         if self._held is not None:
             _need(self._held_route is None, "together(): one routing at most")
             self._held_route = (logits, rargs, (logits, rargs, r, choice_bias))
@@ -1070,6 +1098,137 @@ class HipOps:
         self._gemm(x.view(t * heads, x.shape[2]), w, out.view(t * heads, out.shape[2]),
                    m=t * heads, n=n, k=k, offsets=offsets, a_index=index, c_index=index,
                    groups=heads, w_group_stride=n * k)
+
+    # ---- parallel sublayers, hashed pairs, differential attention ------------------------
+    def embed_pairs(self, ctx, table, out, scale=1.0, pair_table=None, buckets=0, mul_prev=0,
+                    mul_cur=0, state=None):
+        """out[t] = table[token[t]] scale (+ pair_table[row]) in 32-bit, row = (previous token x
+        mul_prev + token x mul_cur) mod buckets, or `buckets` (the table's last row) for a
+        request's first token. The token before a step's first row comes from `state` ([slots,
+        >= 1] 32-bit view: previous token + 1 as an integer, 0 for none), which is moved on to
+        the step's last token."""
+        _dev(table, "table", dims=2)
+        _dev(out, "out", torch.float32, 2)
+        _need(out.shape == (ctx.T, table.shape[1]), "embed_pairs: out has the wrong shape")
+        state_ptr, stride = None, 0
+        if pair_table is not None:
+            _dev(pair_table, "pair_table", table.dtype, 2)
+            _need(pair_table.shape == (buckets + 1, table.shape[1]) and buckets > 0,
+                  "embed_pairs: the table of pairs must have buckets + 1 rows")
+            _need(state is not None and state.is_cuda and state.dtype == torch.float32
+                  and state.dim() == 2 and state.shape[1] >= 1,
+                  "embed_pairs: the state must be 32-bit rows of at least one number")
+            state_ptr, stride = state.data_ptr(), state.stride(0)
+        self._ok(self.lib.ninfer_embed_pairs(
+            ctypes.c_void_p(ctx.tokens.data_ptr()), ctypes.c_void_p(table.data_ptr()),
+            ctypes.c_void_p(out.data_ptr()), ctx.T, table.shape[1], _DT[table.dtype],
+            ctypes.c_float(scale), ctypes.c_void_p(_ptr(pair_table)), int(buckets), int(mul_prev),
+            int(mul_cur), ctypes.c_void_p(ctx.row_seq.data_ptr()),
+            ctypes.c_void_p(ctx.seq_row_start.data_ptr()), ctypes.c_void_p(ctx.seq_slots.data_ptr()),
+            ctx.S, ctypes.c_void_p(state_ptr), ctypes.c_longlong(stride), self._stream()))
+
+    def concat_rows(self, a, b, out):
+        """out[:, :H] = a, out[:, H:] = b (a, b: 32-bit [T, H]; out: [T, 2H] of any dtype)."""
+        _dev(a, "a", torch.float32, 2)
+        _dev(b, "b", torch.float32, 2)
+        _dev(out, "out", dims=2)
+        _need(a.shape == b.shape and out.shape == (a.shape[0], 2 * a.shape[1])
+              and out.dtype in _DT, "concat_rows: shapes")
+        self._ok(self.lib.ninfer_concat_rows(
+            ctypes.c_void_p(a.data_ptr()), ctypes.c_void_p(b.data_ptr()),
+            ctypes.c_void_p(out.data_ptr()), a.shape[0], a.shape[1], _DT[out.dtype], self._stream()))
+
+    def scaled_sum_add(self, residual, a, s1, f, s2):
+        """residual += s1 a + s2 f in 32-bit: a rows [T, H] or None; f rows [T, H], a weighted
+        sum of rows (an object with y, weights, shared, gate) or None; s1, s2 [H] 32-bit or
+        None (factor 1)."""
+        _dev(residual, "residual", torch.float32, 2)
+        t, h = residual.shape
+        dtype = None
+        if a is not None:
+            _dev(a, "a", dims=2)
+            _need(a.shape == (t, h) and a.dtype in _DT, "scaled_sum_add: a does not fit")
+            dtype = a.dtype
+        for name, sc in (("s1", s1), ("s2", s2)):
+            if sc is not None:
+                _dev(sc, name, torch.float32, 1)
+                _need(sc.shape[0] == h, f"scaled_sum_add: {name} has the wrong size")
+        dense = y = w = shared = gate = None
+        k = gs = 0
+        if f is not None and hasattr(f, "weights"):
+            dtype = dtype or f.y.dtype
+            k, gs = self._check_rows_sum(f, t, h, dtype)
+            y, w, shared, gate = f.y.data_ptr(), f.weights.data_ptr(), _ptr(f.shared), _ptr(f.gate)
+        elif f is not None:
+            dtype = dtype or f.dtype
+            _dev(f, "f", dtype, 2)
+            _need(f.shape == (t, h), "scaled_sum_add: f does not fit")
+            dense = f.data_ptr()
+        if dtype is None:
+            return
+        self._ok(self.lib.ninfer_scaled_sum_add(
+            ctypes.c_void_p(residual.data_ptr()), ctypes.c_void_p(_ptr(a)), ctypes.c_void_p(_ptr(s1)),
+            ctypes.c_void_p(dense), ctypes.c_void_p(y), ctypes.c_void_p(w), k,
+            ctypes.c_void_p(shared), ctypes.c_void_p(gate), gs, ctypes.c_void_p(_ptr(s2)), t, h,
+            _DT[dtype], self._stream()))
+
+    def tanh_cap(self, x, cap):
+        """x <- cap tanh(x / cap) in place (32-bit numbers)."""
+        _dev(x, "x", torch.float32)
+        self._ok(self.lib.ninfer_tanh_cap(ctypes.c_void_p(x.data_ptr()),
+                                          ctypes.c_longlong(x.numel()), ctypes.c_float(cap),
+                                          self._stream()))
+
+    def relu_square(self, x):
+        """x <- max(x, 0)^2 in place."""
+        _dev(x, "x")
+        _need(x.dtype in _DT, f"relu_square: tensor of {x.dtype}")
+        self._ok(self.lib.ninfer_relu_square(ctypes.c_void_p(x.data_ptr()),
+                                             ctypes.c_longlong(x.numel()), _DT[x.dtype],
+                                             self._stream()))
+
+    def diff_attention(self, qkv, k_pool, v_pool, block_table, ctx, heads, kv_heads, dim, vdim,
+                       page_size, scale, cap, temp_coef, temp_every, lam, eps, out_scale, out,
+                       write_kv=True):
+        """Differential attention of the rows of `qkv` ([T, heads x 2 dim | kv_heads x 2 dim |
+        kv_heads x vdim]: two queries and two keys per head, [map 1 | map 2], and one value):
+        k and v go into the requests' pages (`write_kv`), then every query head forms
+        a1 - lam a2 from its two causal softmax attentions over the same values, divides it by
+        its root mean square over vdim (eps inside the root; eps < 0: no norm) and multiplies
+        by out_scale. Scores: (q . k) scale (1 + temp_coef ln(floor((p + 1) / temp_every) + 1))
+        at the row's position p, then cap tanh(. / cap) when cap > 0. out: [T, heads x vdim]."""
+        _dev(qkv, "qkv", dims=2)
+        _need(qkv.dtype in _DT, f"diff_attention: rows of {qkv.dtype}")
+        _dev(k_pool, "k_pool", qkv.dtype, 4)
+        _dev(v_pool, "v_pool", qkv.dtype, 4)
+        _dev(out, "out", qkv.dtype, 2)
+        _dev(block_table, "block_table", torch.int32, 2)
+        t = qkv.shape[0]
+        _need(t == ctx.T and qkv.shape[1] == (heads + kv_heads) * 2 * dim + kv_heads * vdim,
+              "diff_attention: qkv has the wrong shape")
+        _need(out.shape == (t, heads * vdim), "diff_attention: out has the wrong shape")
+        _need(k_pool.shape[1:] == (kv_heads, page_size, 2 * dim)
+              and v_pool.shape[1:] == (kv_heads, page_size, vdim)
+              and k_pool.shape[0] == v_pool.shape[0],
+              "diff_attention: pools do not fit the head layout")
+        _need(block_table.shape[0] == ctx.S, "diff_attention: block table rows != requests")
+        a = _DiffAttnArgs()
+        a.qkv, a.kpool, a.vpool, a.out = qkv.data_ptr(), k_pool.data_ptr(), v_pool.data_ptr(), out.data_ptr()
+        a.block_table, a.positions = block_table.data_ptr(), ctx.positions.data_ptr()
+        a.row_seq, a.seq_row_start = ctx.row_seq.data_ptr(), ctx.seq_row_start.data_ptr()
+        a.q_stride, a.bt_stride, a.T, a.S = qkv.shape[1], block_table.shape[1], t, ctx.S
+        a.Hq, a.Hkv, a.dim, a.vdim, a.page_size = heads, kv_heads, dim, vdim, page_size
+        a.dtype, a.max_qlen, a.max_kv_len = _DT[qkv.dtype], ctx.max_qlen, ctx.max_kv_len
+        a.force_plain = 1 if self.force_generic else 0
+        a.scale, a.cap, a.t_coef, a.t_every = scale, cap, temp_coef, int(temp_every)
+        a.lam, a.eps, a.out_scale = lam, eps, out_scale
+        if write_kv:
+            self._ok(self.lib.ninfer_diff_kv_write(ctypes.byref(a), self._stream()))
+        need = int(self.lib.ninfer_diff_attention_workspace_floats(ctypes.byref(a)))
+        if need:   # contexts cut into chunks: partial sums, merged by a second kernel
+            ws = self._workspace(need, qkv.device)
+            a.workspace, a.workspace_floats = ws.data_ptr(), ws.numel()
+        self._ok(self.lib.ninfer_diff_attention(ctypes.byref(a), self._stream()))
 
     # ---- sampling -------------------------------------------------------------------
     FEW_TOKENS = 64   # most tokens a row may keep (top_k) for the two-launch sampling path

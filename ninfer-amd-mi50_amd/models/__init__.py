@@ -1,5 +1,6 @@
 from . import getodra  # registers Getodra
 from . import qwen2_moe  # registers Qwen2MoeForCausalLM
+from . import sosepel  # registers Sosepel
 from .spec import LayerCall, ModelSpec
 
-__all__ = ["LayerCall", "ModelSpec", "getodra", "qwen2_moe"]
+__all__ = ["LayerCall", "ModelSpec", "getodra", "qwen2_moe", "sosepel"]

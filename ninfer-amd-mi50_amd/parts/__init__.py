@@ -1,18 +1,21 @@
 from .attention import Attention
 from .base import (Block, CacheNeed, CacheView, CallInfo, FeedForward, Mixer, Norm, Part,
                    PendingRows, PoolSpec, PositionEncoding, StepContext, WeightBinder, settle)
-from .block import OutputNormBlock, PreNormBlock
+from .block import OutputNormBlock, ParallelBlock, PreNormBlock
+from .diff_attention import DifferentialAttention
 from .embedding import LMHead, TokenEmbedding
 from .latent_attention import LatentAttention
 from .lightning import LightningAttention
-from .mlp import SwiGLU
+from .mlp import MLP, SwiGLU
 from .moe import RoutedExperts, Routing, SoftmaxTopKRouter, SparseMoE, TopKRouter
 from .norm import OutputRMSNorm, RMSNorm
 from .rotary import NoPosition, Rotary
+from .reentry import StreamReentry
 from .short_conv import ShortConv
 
 __all__ = ["Attention", "Block", "CacheNeed", "CacheView", "CallInfo", "FeedForward", "Mixer",
            "Norm", "Part", "PendingRows", "PoolSpec", "settle", "PositionEncoding", "StepContext", "WeightBinder", "PreNormBlock",
            "LMHead", "TokenEmbedding", "SwiGLU", "RoutedExperts", "Routing", "SoftmaxTopKRouter", "TopKRouter",
            "SparseMoE", "RMSNorm", "NoPosition", "Rotary", "OutputNormBlock", "OutputRMSNorm",
-           "LatentAttention", "LightningAttention", "ShortConv"]
+           "LatentAttention", "LightningAttention", "ShortConv", "ParallelBlock",
+           "DifferentialAttention", "MLP", "StreamReentry"]

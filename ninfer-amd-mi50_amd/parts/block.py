@@ -11,7 +11,11 @@ from __future__ import annotations
 from typing import List, Optional
 
 from ..registry import register_part
-from .base import Block, CallInfo, FeedForward, Mixer, Norm, Part, StepContext, settle
+import torch
+
+from ..weights.source import TensorSpec
+from .base import (Block, CallInfo, FeedForward, Mixer, Norm, Part, PendingRows, StepContext,
+                   WeightBinder, settle)
 
 
 class PreNormBlock(Block):
@@ -92,3 +96,52 @@ class OutputNormBlock(Block):
 
 
 register_part("block", "output_norm", OutputNormBlock)
+
+
+class ParallelBlock(Block):
+    """A block whose sublayers read the same normed rows: h = norm(x), then
+    x += s1 mixer(h) + s2 feed_forward(h), with s1 and s2 one learned factor per column
+    (`mixer_scale`, `ff_scale`: tensor names, None for no factor). `feed_forward` may be None.
+    The sum is formed in 32-bit by one kernel, which also adds up a sparse feed-forward's
+    weighted rows."""
+
+    def __init__(self, norm: Norm, mixer: Mixer, feed_forward: Optional[FeedForward] = None,
+                 mixer_scale: Optional[str] = None, ff_scale: Optional[str] = None, size: int = 0):
+        self.norm = norm
+        self.mixer = mixer
+        self.feed_forward = feed_forward
+        self.mixer_scale_name = mixer_scale
+        self.ff_scale_name = ff_scale if feed_forward is not None else None
+        self.spare_scale_name = ff_scale if feed_forward is None else None
+        self.size = size
+        self.mixer_scale: Optional[torch.Tensor] = None
+        self.ff_scale: Optional[torch.Tensor] = None
+
+    def children(self) -> List[Part]:
+        return [p for p in (self.norm, self.mixer, self.feed_forward) if p is not None]
+
+    def tensor_specs(self):
+        return {n: TensorSpec((self.size,), "gain")
+                for n in (self.mixer_scale_name, self.ff_scale_name) if n}
+
+    def unused_tensor_specs(self):
+        # a layer without a feed-forward may still carry the factor of one
+        if self.spare_scale_name:
+            return {self.spare_scale_name: TensorSpec((self.size,), "gain")}
+        return {}
+
+    def bind(self, w: WeightBinder) -> None:
+        if self.mixer_scale_name:
+            self.mixer_scale = w.float32(self.mixer_scale_name)
+        if self.ff_scale_name:
+            self.ff_scale = w.float32(self.ff_scale_name)
+
+    def forward(self, ctx: StepContext, residual, pending, call: CallInfo):
+        h = self.norm.forward(ctx, residual, pending)
+        a = self.mixer.forward(ctx, h, residual, call)
+        f = self.feed_forward.forward(ctx, h, residual) if self.feed_forward is not None else None
+        ctx.ops.scaled_sum_add(residual, a, self.mixer_scale, f, self.ff_scale)
+        return None
+
+
+register_part("block", "parallel", ParallelBlock)

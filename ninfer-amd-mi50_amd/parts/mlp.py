@@ -79,3 +79,41 @@ class SwiGLU(FeedForward):
 
 
 register_part("feed_forward", "swiglu", SwiGLU)
+
+
+class MLP(FeedForward):
+    """Dense feed-forward without a gate: act(x Wu^T) Wd^T, no biases. `act`: 'relu2', the
+    square of relu. `names`: what follows the prefix in the names of the two weights."""
+
+    ACTS = ("relu2",)
+
+    def __init__(self, prefix: str, hidden: int, inner: int, act: str = "relu2",
+                 names=("up", "down")):
+        if act not in self.ACTS:
+            raise ValueError(f"activation {act!r} is not one of {self.ACTS}")
+        self.prefix = prefix
+        self.names = tuple(names)
+        self.hidden = hidden
+        self.inner = inner
+        self.act = act
+        self.w_up: Optional[torch.Tensor] = None
+        self.w_down: Optional[torch.Tensor] = None
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        p = self.prefix
+        return {p + self.names[0]: TensorSpec((self.inner, self.hidden)),
+                p + self.names[1]: TensorSpec((self.hidden, self.inner))}
+
+    def bind(self, w: WeightBinder) -> None:
+        self.w_up = w.matrix(self.prefix + self.names[0])
+        self.w_down = w.matrix(self.prefix + self.names[1])
+
+    def forward(self, ctx: StepContext, x, residual):
+        h = ctx.empty((x.shape[0], self.inner))
+        ctx.ops.linear(x, self.w_up, h, act=self.act)
+        out = ctx.empty((x.shape[0], self.hidden))
+        ctx.ops.linear(h, self.w_down, out)
+        return out
+
+
+register_part("feed_forward", "mlp", MLP)

@@ -33,7 +33,11 @@ class TopKRouter(Part):
 
     def __init__(self, prefix: str, hidden: int, experts: int, top_k: int, renorm: bool,
                  score: str = "softmax", scale: float = 1.0, choice_bias: bool = False,
-                 n_group: int = 0, topk_group: int = 0):
+                 n_group: int = 0, topk_group: int = 0, group_top: int = 1,
+                 renorm_eps: float = 0.0, leaf: str = "weight"):
+        """`group_top`: a group's score in the group-limited choice is the sum of its group_top
+        largest scores (1: its largest). `renorm_eps` is added to the sum of the chosen scores
+        before the division. `leaf`: what follows the prefix in the weight's name."""
         if top_k > experts:
             raise ValueError(f"top_k ({top_k}) exceeds the number of experts ({experts})")
         if score not in ("softmax", "sigmoid"):
@@ -49,6 +53,9 @@ class TopKRouter(Part):
         # a group-limited choice: only the experts of the topk_group groups (of experts /
         # n_group neighbours each) whose best score (+ bias) is largest are candidates
         self.n_group, self.topk_group = int(n_group), int(topk_group)
+        self.group_top, self.renorm_eps, self.leaf = int(group_top), float(renorm_eps), leaf
+        if self.n_group > 1 and not 1 <= self.group_top <= experts // max(1, self.n_group):
+            raise ValueError(f"group_top ({self.group_top}) must lie in [1, experts per group]")
         if self.n_group > 1 and (experts % self.n_group or not 1 <= self.topk_group <= self.n_group
                                  or self.topk_group * (experts // self.n_group) < top_k):
             raise ValueError(f"{self.n_group} groups of which {self.topk_group} are open do not fit "
@@ -57,13 +64,13 @@ class TopKRouter(Part):
         self.choice_bias: Optional[torch.Tensor] = None
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
-        specs = {self.prefix + "weight": TensorSpec((self.experts, self.hidden))}
+        specs = {self.prefix + self.leaf: TensorSpec((self.experts, self.hidden))}
         if self.has_choice_bias:
             specs[self.prefix + "choice_bias"] = TensorSpec((self.experts,), role="bias")
         return specs
 
     def bind(self, w: WeightBinder) -> None:
-        self.weight = w.matrix(self.prefix + "weight")
+        self.weight = w.matrix(self.prefix + self.leaf)
         if self.has_choice_bias:
             self.choice_bias = w.float32(self.prefix + "choice_bias")
 
@@ -84,7 +91,8 @@ class TopKRouter(Part):
                     tile_counts=ctx.empty((2,), torch.int32))
         ctx.ops.moe_route(logits, e, k, self.renorm, r, score=self.score,
                           choice_bias=self.choice_bias, scale=self.scale, n_group=self.n_group,
-                          topk_group=self.topk_group)
+                          topk_group=self.topk_group, group_top=self.group_top,
+                          renorm_eps=self.renorm_eps)
         return r
 
 
@@ -111,7 +119,11 @@ class RoutedExperts(Part):
     """E SwiGLU experts with stacked weights [E, 2I, hidden] and [E, hidden, I]
     built from the per-expert checkpoint tensors `experts.{e}.*_proj.weight`."""
 
-    def __init__(self, prefix: str, hidden: int, inner: int, experts: int, act: str = "silu"):
+    def __init__(self, prefix: str, hidden: int, inner: int, experts: int, act: str = "silu",
+                 names=("gate_proj.weight", "up_proj.weight", "down_proj.weight")):
+        """`names`: what follows `prefix + str(e) + "."` in the names of expert e's gate, other
+        half and down weights."""
+        self.names = tuple(names)
         self.prefix = prefix
         self.hidden = hidden
         self.inner = inner
@@ -124,9 +136,9 @@ class RoutedExperts(Part):
         specs = {}
         for e in range(self.experts):
             p = f"{self.prefix}{e}."
-            specs[p + "gate_proj.weight"] = TensorSpec((self.inner, self.hidden))
-            specs[p + "up_proj.weight"] = TensorSpec((self.inner, self.hidden))
-            specs[p + "down_proj.weight"] = TensorSpec((self.hidden, self.inner))
+            specs[p + self.names[0]] = TensorSpec((self.inner, self.hidden))
+            specs[p + self.names[1]] = TensorSpec((self.inner, self.hidden))
+            specs[p + self.names[2]] = TensorSpec((self.hidden, self.inner))
         return specs
 
     def bind(self, w: WeightBinder) -> None:
@@ -137,9 +149,9 @@ class RoutedExperts(Part):
                                   device=w.device)
         for e in range(self.experts):
             p = f"{self.prefix}{e}."
-            w.matrix_into(p + "gate_proj.weight", self.w_gate_up[e, :i])
-            w.matrix_into(p + "up_proj.weight", self.w_gate_up[e, i:])
-            w.matrix_into(p + "down_proj.weight", self.w_down[e])
+            w.matrix_into(p + self.names[0], self.w_gate_up[e, :i])
+            w.matrix_into(p + self.names[1], self.w_gate_up[e, i:])
+            w.matrix_into(p + self.names[2], self.w_down[e])
 
     def gate_up(self, ctx: StepContext, x: torch.Tensor, routing: "Routing") -> torch.Tensor:
         """Activations [T*k, inner] in sorted order (row r belongs to the expert that
@@ -161,17 +173,30 @@ class RoutedExperts(Part):
 
 
 class SparseMoE(FeedForward):
+    # what follows the prefix in the tensors' names, by default (a model with other names
+    # passes `names` with the entries that differ)
+    NAMES = {"router": "gate.", "router_leaf": "weight", "experts": "experts.",
+             "expert_leaves": ("gate_proj.weight", "up_proj.weight", "down_proj.weight"),
+             "shared": "shared_expert.", "shared_gate": "shared_expert_gate.weight"}
+
     def __init__(self, prefix: str, hidden: int, experts: int, top_k: int, inner: int,
-                 renorm: bool, shared_inner: int = 0, act: str = "silu"):
+                 renorm: bool, shared_inner: int = 0, act: str = "silu", router=None, names=None):
+        """`router`: further parameters of `TopKRouter` (score, scale, n_group, topk_group,
+        group_top, renorm_eps, choice_bias)."""
         self.prefix = prefix
         self.hidden = hidden
-        self.router = SoftmaxTopKRouter(prefix + "gate.", hidden, experts, top_k, renorm)
-        self.experts = RoutedExperts(prefix + "experts.", hidden, inner, experts, act)
+        n = dict(self.NAMES, **(names or {}))
+        self.names = n
+        self.router = TopKRouter(prefix + n["router"], hidden, experts, top_k, renorm,
+                                 leaf=n["router_leaf"], **(router or {}))
+        self.experts = RoutedExperts(prefix + n["experts"], hidden, inner, experts, act,
+                                     names=n["expert_leaves"])
         self.shared: Optional[SwiGLU] = None
         self.shared_gate: Optional[torch.Tensor] = None
         self.last_ids: Optional[torch.Tensor] = None   # routing of the last step (for statistics)
         if shared_inner > 0:
-            self.shared = SwiGLU(prefix + "shared_expert.", hidden, shared_inner, act)
+            self.shared = SwiGLU(prefix + n["shared"], hidden, shared_inner, act,
+                                 names=n["expert_leaves"])
 
     def children(self) -> List[Part]:
         return [self.router, self.experts] + ([self.shared] if self.shared else [])
@@ -179,11 +204,11 @@ class SparseMoE(FeedForward):
     def tensor_specs(self) -> Dict[str, TensorSpec]:
         if self.shared is None:
             return {}
-        return {self.prefix + "shared_expert_gate.weight": TensorSpec((1, self.hidden))}
+        return {self.prefix + self.names["shared_gate"]: TensorSpec((1, self.hidden))}
 
     def bind(self, w: WeightBinder) -> None:
         if self.shared is not None:
-            self.shared_gate = w.matrix(self.prefix + "shared_expert_gate.weight")
+            self.shared_gate = w.matrix(self.prefix + self.names["shared_gate"])
 
     def bind_all(self, w: WeightBinder) -> None:
         super().bind_all(w)
@@ -193,8 +218,8 @@ class SparseMoE(FeedForward):
             self.router_and_gate = torch.cat([self.router.weight, self.shared_gate])
             self.router.weight = self.router_and_gate[:e]
             self.shared_gate = self.router_and_gate[e:]
-            w.hold(self.router.prefix + "weight", self.router.weight)
-            w.hold(self.prefix + "shared_expert_gate.weight", self.shared_gate)
+            w.hold(self.router.prefix + self.router.leaf, self.router.weight)
+            w.hold(self.prefix + self.names["shared_gate"], self.shared_gate)
 
     def forward(self, ctx: StepContext, x, residual):
         if self.shared is None:
