@@ -118,10 +118,13 @@ class PlainOps:
             acc = acc + g * _f(shared)
         residual += acc
 
-    def linear(self, x, w, out, bias=None):
+    def linear(self, x, w, out, bias=None, act=None):
         r = _f(x) @ _f(w).T
         if bias is not None:
             r = r + bias
+        if act is not None:
+            assert act == "relu2", act
+            r = torch.relu(r) ** 2
         out.copy_(r.to(out.dtype))
 
     @staticmethod
@@ -162,7 +165,8 @@ class PlainOps:
             out[rows] = (_f(h[off[g]:off[g + 1]]) @ _f(w_down[g]).T).to(out.dtype)
 
     def router_topk(self, logits, experts, top_k, renorm, ids, wts, score="softmax",
-                    choice_bias=None, scale=1.0, n_group=0, topk_group=0):
+                    choice_bias=None, scale=1.0, n_group=0, topk_group=0, group_top=1,
+                    renorm_eps=0.0):
         l = logits[:, :experts]
         if score == "sigmoid":
             p = 1 / (1 + torch.exp(-l))
@@ -174,7 +178,8 @@ class PlainOps:
         if n_group > 1 and topk_group < n_group:
             # group-limited: the groups by their best score, a stable sort (ties: lower group)
             per = experts // n_group
-            best_of = work.view(-1, n_group, per).max(-1).values
+            # (a group's score: its best, or the sum of its group_top best)
+            best_of = work.view(-1, n_group, per).topk(max(1, group_top), -1).values.sum(-1)
             keep = torch.sort(best_of, dim=-1, descending=True, stable=True).indices[:, :topk_group]
             is_open = torch.zeros_like(best_of, dtype=torch.bool)
             is_open.scatter_(1, keep, True)
@@ -187,7 +192,7 @@ class PlainOps:
             wts[:, j] = p[rows, idx]
             work[rows, idx] = -float("inf")
         if renorm:
-            wts /= wts.sum(-1, keepdim=True)
+            wts /= wts.sum(-1, keepdim=True) + renorm_eps
         wts *= scale
 
     def moe_align(self, ids, experts, offsets, order, tiles=None):
@@ -206,9 +211,9 @@ class PlainOps:
                 tiles.tile_counts[0 if size == 16 else 1] = len(lst)
 
     def moe_route(self, logits, experts, top_k, renorm, r, score="softmax", choice_bias=None,
-                  scale=1.0, n_group=0, topk_group=0):
+                  scale=1.0, n_group=0, topk_group=0, group_top=1, renorm_eps=0.0):
         self.router_topk(logits, experts, top_k, renorm, r.ids, r.weights, score, choice_bias,
-                         scale, n_group, topk_group)
+                         scale, n_group, topk_group, group_top, renorm_eps)
         self.moe_align(r.ids, experts, r.offsets, r.order, tiles=r)
 
     def paged_attention(self, qkv, k_pool, v_pool, block_table, ctx, n_q, n_kv, head_dim,
@@ -233,6 +238,78 @@ class PlainOps:
                 p = torch.exp(s - s.max())
                 p = p / p.sum()
                 out[r, h * head_dim:(h + 1) * head_dim] = (p @ v[:, g, :]).to(out.dtype)
+
+    # ---- parallel sublayers, hashed pairs, differential attention ------------------------------
+    def embed_pairs(self, ctx, table, out, scale=1.0, pair_table=None, buckets=0, mul_prev=0,
+                    mul_cur=0, state=None):
+        toks = ctx.tokens.tolist()
+        x = _f(table[ctx.tokens.long()]) * scale
+        if pair_table is not None:
+            start, slots = ctx.seq_row_start.tolist(), ctx.seq_slots.tolist()
+            held = state.view(torch.int32)
+            for s in range(ctx.S):
+                prev = int(held[slots[s], 0]) - 1
+                for t in range(start[s], start[s + 1]):
+                    row = buckets if prev < 0 else (prev * mul_prev + toks[t] * mul_cur) % buckets
+                    x[t] += _f(pair_table[row])
+                    prev = toks[t]
+                held[slots[s], 0] = prev + 1
+        out.copy_(x)
+
+    def concat_rows(self, a, b, out):
+        out.copy_(torch.cat([a, b], -1).to(out.dtype))
+
+    def scaled_sum_add(self, residual, a, s1, f, s2):
+        if a is not None:
+            residual += _f(a) * (s1 if s1 is not None else 1.0)
+        if f is None:
+            return
+        if hasattr(f, "weights"):
+            add = torch.zeros_like(residual)
+            self.moe_combine(add, f.y, f.weights, f.shared, f.gate)
+        else:
+            add = _f(f)
+        residual += add * (s2 if s2 is not None else 1.0)
+
+    def tanh_cap(self, x, cap):
+        x.copy_(cap * torch.tanh(x / cap))
+
+    def relu_square(self, x):
+        x.copy_((torch.relu(_f(x)) ** 2).to(x.dtype))
+
+    def diff_attention(self, qkv, k_pool, v_pool, block_table, ctx, heads, kv_heads, dim, vdim,
+                       page_size, scale, cap, temp_coef, temp_every, lam, eps, out_scale, out,
+                       write_kv=True):
+        t = qkv.shape[0]
+        nq, nk = heads * 2 * dim, kv_heads * 2 * dim
+        pos, seq = ctx.positions.tolist(), ctx.row_seq.tolist()
+        if write_kv:
+            for r in range(t):
+                page = int(block_table[seq[r], pos[r] // page_size])
+                assert page >= 0, "write into a page that is not held"
+                k_pool[page, :, pos[r] % page_size] = qkv[r, nq:nq + nk].view(kv_heads, 2 * dim)
+                v_pool[page, :, pos[r] % page_size] = qkv[r, nq + nk:].view(kv_heads, vdim)
+        q = _f(qkv[:, :nq]).view(t, heads, 2, dim)
+        for r in range(t):
+            js = torch.arange(0, pos[r] + 1)
+            pages = block_table[seq[r], js // page_size].long()
+            assert (pages >= 0).all(), "read of a page that is not held"
+            k = _f(k_pool[pages, :, js % page_size]).view(-1, kv_heads, 2, dim)
+            v = _f(v_pool[pages, :, js % page_size])
+            temp = 1.0 + temp_coef * math.log((pos[r] + 1) // temp_every + 1) if temp_coef else 1.0
+            for h in range(heads):
+                g = h // (heads // kv_heads)
+                maps = []
+                for i in range(2):
+                    s = (k[:, g, i] @ q[r, h, i]) * (scale * temp)
+                    if cap > 0:
+                        s = cap * torch.tanh(s / cap)
+                    p = torch.exp(s - s.max())
+                    maps.append((p / p.sum()) @ v[:, g])
+                o = maps[0] - lam * maps[1]
+                if eps >= 0:
+                    o = o / torch.sqrt((o * o).mean() + eps)
+                out[r, h * vdim:(h + 1) * vdim] = (o * out_scale).to(out.dtype)
 
     def sample(self, logits, temperature, uniform, out, top_k=None, top_p=None, rep_penalty=None,
                pen_tokens=None, pen_counts=None, pen_offsets=None):

@@ -113,3 +113,92 @@ def test_plain_pair_rows_and_temperature():
     assert plain_sosepel.pair_rows([3, 4, 4], 7, 5, 2) == [7, (15 + 8) % 7, (20 + 8) % 7]
     t = plain_sosepel.query_temperature(9, {"coef": 0.5, "every": 4})
     assert t[2] == 1.0 and t[3] == 1.0 + 0.5 * math.log(2) and t[6] == t[3] and t[7] == 1.0 + 0.5 * math.log(3)
+
+
+# ---- the engine's host logic on the CPU, with plain stand-ins for the kernels ------------------
+
+@pytest.fixture(scope="module", params=["odd", "ones", "straight"])
+def host_case(request, tmp_path_factory):
+    import ninfer_amd
+    make, seed = sosepel_cases.CASES[request.param]
+    raw = make()
+    d = str(tmp_path_factory.mktemp("sosepel_host_" + request.param))
+    ninfer_amd.write_random_model(d, raw, seed, dtype="float32", std=0.25)
+    cfg, w = util.read_folder(d)
+    reqs = {f"r{i}": util.random_tokens(n, raw["vocab"], 20 + i) for i, n in enumerate([33, 1, 12, 47, 20])}
+    margins = {k: [] for k in reqs}
+    ref = {k: plain_sosepel.forward(w, cfg, v, margins=margins[k]) for k, v in reqs.items()}
+    # rows at which a routing decision is a close call are left out of the comparisons
+    clear = {k: torch.stack([m > 1e-4 for m in margins[k]]).all(0) if margins[k]
+             else torch.ones(len(reqs[k]), dtype=torch.bool) for k in reqs}
+    return {"dir": d, "cfg": raw, "reqs": reqs, "ref": ref, "clear": clear}
+
+
+def _host_runner(case, **more):
+    from ninfer_amd import EngineOptions, load_model
+    from plain_ops import PlainOps
+    opt = dict(dtype="float32", device="cpu", max_context=64, num_sequences=4, page_size=4, num_pages=40,
+               check_pages=True)
+    opt.update(more)
+    return load_model(case["dir"], EngineOptions(**opt), ops=PlainOps())
+
+
+def _close(case, got):
+    for rid, g in got.items():
+        rid = rid.split("#")[0]
+        ok = case["clear"][rid]
+        # a close call at one row changes what that row writes into the cache for all later rows
+        upto = int((~ok).nonzero()[0]) if (~ok).any() else len(ok)
+        torch.testing.assert_close(g.double()[:upto], case["ref"][rid][:upto], atol=2e-4, rtol=2e-4)
+
+
+def test_host_every_way_of_cutting(host_case):
+    runner = _host_runner(host_case)
+    for rid, toks in host_case["reqs"].items():
+        scheds = [util.schedule_whole(rid, toks), util.schedule_portions(rid, toks, seed=len(toks))]
+        if len(toks) > 1:
+            scheds.append(util.schedule_tail(rid, toks, 9))
+        for sched in scheds:
+            _close(host_case, util.run_schedule(runner, sched))
+    assert all(g.allocator.in_use == 0 for g in runner.cache.groups)
+
+
+def test_host_mixed_batches_reuse_pages_and_slots(host_case):
+    """Portions beside single tokens, a pool that forces pages to be used again, two state
+    slots for five requests and their repeats: a slot's previous token is that of its request."""
+    runner = _host_runner(host_case, num_sequences=2, num_pages=26)
+    reqs = dict(host_case["reqs"])
+    reqs.update({k + "#2": v for k, v in host_case["reqs"].items()})
+    _close(host_case, util.run_schedule(runner, util.schedule_mixed(reqs, seed=2, max_live=2)))
+    assert runner.cache.pages_reused() > 0
+    runner.cache.check()
+
+
+def test_host_generation_through_the_scheduler(host_case):
+    """Greedy generation by the scheduler (admission, portions under a token budget, batched
+    decoding with fewer slots than requests), token for token the plain choice. Preemption
+    gives a request's slot to another and runs it again from its first token."""
+    from ninfer_amd import Request, Sampler, SamplingParams, Scheduler
+    from plain_ops import PlainOps
+    cfg, w = util.read_folder(host_case["dir"])
+    prompts = [host_case["reqs"]["r2"], host_case["reqs"]["r1"], host_case["reqs"]["r4"][:7],
+               host_case["reqs"]["r0"][:15]]
+    want = []
+    for p in prompts:
+        toks = list(p)
+        for _ in range(6):
+            margins = []
+            logits = plain_sosepel.forward(w, cfg, toks, margins=margins)[-1]
+            top = torch.topk(logits, 2).values
+            if top[0] - top[1] < 1e-3 or any(float(m.min()) < 1e-3 for m in margins):
+                break
+            toks.append(int(logits.argmax()))
+        want.append(toks[len(p):])
+    runner = _host_runner(host_case, num_sequences=2, prefill_chunk=8, num_pages=14)
+    sched = Scheduler(runner, Sampler(PlainOps(), runner.device))
+    reqs = [Request(f"q{i}", list(p), SamplingParams.greedy(6)) for i, p in enumerate(prompts)]
+    for r in reqs:
+        sched.add(r)
+    sched.run()
+    assert all(r.status == "finished" for r in reqs), [r.error for r in reqs]
+    assert [r.output[:len(x)] for r, x in zip(reqs, want)] == want
