@@ -23,6 +23,12 @@ lightning attention layers with input convolutions and output norms) beside a de
 Qwen2-style model of the same width, depth, heads and feed-forward size, both with random
 weights: prompt portions of 512 and 2,048 tokens and decode steps at batch 1, 8 and 64.
 
+    python bench.py --scenario designs --design sosepel [--sizes small,medium] [--only sosepel|sparse]
+
+runs the same measurement for Sosepel (parallel blocks of differential attention and a dense or
+sparse feed-forward, a hashed pair embedding, layers that run twice) beside a Qwen2-MoE model of
+the same width, heads and experts with as many layers as the other has layer runs.
+
     python bench.py --scenario long [--model 57b-a14b] [--requests 8] [--prompt 32768] [--new 256]
 
 is another measurement with a JSON line of its own: the scheduler serves
@@ -85,6 +91,9 @@ def main() -> int:
     ap.add_argument("--scenario", default="decode", choices=["decode", "long", "designs"])
     ap.add_argument("--sizes", default="small,medium",
                     help="--scenario designs: which of the layer sizes to run (small, medium)")
+    ap.add_argument("--design", default="getodra", choices=["getodra", "sosepel"],
+                    help="--scenario designs: the design to run beside the closest model the engine had")
+    ap.add_argument("--only", default="", help="--scenario designs: run this one of the two models only")
     ap.add_argument("--requests", type=int, default=8, help="--scenario long: concurrent requests")
     ap.add_argument("--prompt", type=int, default=32768, help="--scenario long: prompt tokens")
     ap.add_argument("--new", type=int, default=256, help="--scenario long: new tokens a request")
@@ -507,19 +516,67 @@ def dense_config(z: dict) -> dict:
                 hidden_act="gelu_pytorch_tanh")
 
 
+SOSEPEL_SIZES = {
+    # width, dense feed-forward, layers (layers 1 .. layers - 2 run twice), query and kv heads,
+    # sizes of a map's query and key and of a value, experts
+    "small": dict(width=1024, ff=2816, layers=5, heads=8, kv_heads=2, dim=64, vdim=128, experts=16,
+                  top=2, groups=(4, 2), expert_ff=704, shared_ff=1408, vocab=32000, positions=4096),
+    "medium": dict(width=2048, ff=5632, layers=6, heads=16, kv_heads=4, dim=64, vdim=128, experts=32,
+                   top=4, groups=(4, 2), expert_ff=1408, shared_ff=2816, vocab=32000, positions=4096),
+}
+
+
+def sosepel_config(z: dict) -> dict:
+    """A dense first layer, then sparse ones; the layers between the first and the last run
+    twice, each run with a cache of its own."""
+    mixer = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["vdim"],
+             "diff": 0.6, "scale": z["dim"] ** -0.5, "softcap": 50.0, "q_temp": {"coef": 0.3, "every": 64}}
+    moe = {"kind": "moe", "expert": {"ff": z["expert_ff"]}, "shared": {"ff": z["shared_ff"]},
+           "router": {"experts": z["experts"], "top": z["top"],
+                      "groups": {"count": z["groups"][0], "keep": z["groups"][1]}}}
+    layers = [{"type": "attention", "mixer": mixer, "mlp": {"kind": "dense", "ff": z["ff"]}}]
+    layers += [{"type": "attention", "mixer": mixer, "mlp": moe} for _ in range(z["layers"] - 1)]
+    return {"architecture": "Sosepel", "vocab": z["vocab"], "width": z["width"], "norm": {"eps": 1e-6},
+            "logit_softcap": 15.0, "embedding": {"scale": 0.5, "bigram": {"buckets": 65521, "mul_prev": 127,
+                                                                         "mul_cur": 7}},
+            "layers": layers, "loop": {"start": 1, "stop": z["layers"] - 1, "times": 2}}
+
+
+def sosepel_runs(z: dict) -> int:
+    return 2 * z["layers"] - 2
+
+
+def sparse_config(z: dict) -> dict:
+    """The closest model the engine had: Qwen2-MoE blocks (rotary attention with as many query
+    and kv heads, heads of 2 x dim; routed experts beside a gated shared expert) of the same
+    width, as many layers as the other model has layer runs, the first one dense."""
+    return dict(CONFIG_C, num_hidden_layers=sosepel_runs(z), hidden_size=z["width"],
+                num_attention_heads=z["heads"], num_key_value_heads=z["kv_heads"], head_dim=2 * z["dim"],
+                intermediate_size=z["ff"], num_experts=z["experts"], num_experts_per_tok=z["top"],
+                moe_intermediate_size=z["expert_ff"], shared_expert_intermediate_size=z["shared_ff"],
+                mlp_only_layers=[0], decoder_sparse_step=1, vocab_size=z["vocab"], hidden_act="silu",
+                use_sliding_window=False)
+
+
 def designs_scenario(args) -> int:
     import torch
     from ninfer_amd import Chunk, EngineOptions, random_model
+    sosepel = args.design == "sosepel"
 
     gen = torch.Generator().manual_seed(11)
-    out = {"metric": "prefill and decode throughput, Getodra beside a dense model of equal size",
+    out = {"metric": "prefill and decode throughput, " + ("Sosepel beside a Qwen2-MoE model" if sosepel
+                     else "Getodra beside a dense model") + " of equal size",
            "unit": "tok/s", "n_gpus": 1, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
            "data": "synthetic", "sizes": {}}
     for size in args.sizes.split(","):
-        z = DESIGN_SIZES[size]
+        z = (SOSEPEL_SIZES if sosepel else DESIGN_SIZES)[size]
         ctx = z["positions"]
         row = {"shape": z}
-        for name, raw in (("getodra", getodra_config(z)), ("dense", dense_config(z))):
+        pairs = (("sosepel", sosepel_config(z)), ("sparse", sparse_config(z))) if sosepel else \
+            (("getodra", getodra_config(z)), ("dense", dense_config(z)))
+        for name, raw in pairs:
+            if args.only and name != args.only:
+                continue
             opt = EngineOptions(dtype=args.dtype, max_context=ctx, prefill_chunk=2048,
                                 num_sequences=64, page_size=16, use_graph=args.graph)
             runner = random_model(raw, 99, opt)

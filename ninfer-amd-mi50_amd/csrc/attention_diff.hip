@@ -197,6 +197,207 @@ __global__ __launch_bounds__(64) void diff_attention_merge_kernel(DiffAttnArgs a
   diff_finish<T>(a, acc1, acc2, l1, l2, (T*)a.out + ((int64_t)t * a.Hq + h) * a.vdim, lane);
 }
 
+// Single rows (decode steps) in bfloat16: a block of four waves owns one row, HB query heads of
+// one kv head and one chunk of the context, so that keys and values are read once for all of
+// these heads. The waves take the chunk's tiles of 64 keys in turn. Per tile a lane owns a
+// key: its row is loaded in 16-byte pieces and multiplied with the queries of all HB heads and
+// both maps (32-bit, from LDS); the online softmax of each head and map runs across the wave;
+// then a lane owns value columns lane + 64 v and adds up p x value over the tile's keys for
+// every head and map. The waves' sums are put together through LDS, and the block writes the
+// result (one chunk) or its partial sums (the merge kernel's format).
+template <int HB, int VPL>
+__global__ __launch_bounds__(256) void diff_attention_rows_kernel(DiffAttnArgs a, int chunk,
+                                                                  int n_chunks) {
+  constexpr int HM = 2 * HB;   // (head, map) pairs
+  extern __shared__ float smem[];
+  const int kd = 2 * a.dim, dim = a.dim, vdim = a.vdim;
+  float* q_s = smem;                                   // [HB][2 dim]
+  float* p_s = q_s + HB * kd;                          // [4][HM][64]
+  float* ml_s = p_s + 4 * HM * 64;                     // [4][HM][2]
+  float* acc_s = ml_s + 4 * HM * 2;                    // [4][HM][VPL * 64]
+  int64_t* off_s = (int64_t*)(acc_s + 4 * HM * VPL * 64);   // [4][64]
+
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int t = blockIdx.x, c = blockIdx.z;
+  const int hpg = a.Hq / a.Hkv;
+  const int g = blockIdx.y / (hpg / HB);
+  const int h0 = g * hpg + (blockIdx.y % (hpg / HB)) * HB;
+  const int pos = a.positions[t];
+  const int* bt = a.block_table + (int64_t)a.row_seq[t] * a.bt_stride;
+  const int first = n_chunks > 1 ? c * chunk : 0;
+  const int last = n_chunks > 1 ? min(pos, first + chunk - 1) : pos;
+  const float qscale = a.scale * query_temperature(pos, a.t_coef, a.t_every);
+  const bf16* kpool = (const bf16*)a.kpool;
+  const bf16* vpool = (const bf16*)a.vpool;
+
+  const bf16* qr = (const bf16*)a.qkv + (int64_t)t * a.q_stride + h0 * kd;
+  for (int i = tid; i < HB * kd; i += 256) q_s[i] = to_f32(qr[i]);
+  __syncthreads();
+
+  float m[HM], l[HM], acc[HM][VPL];
+#pragma unroll
+  for (int i = 0; i < HM; ++i) {
+    m[i] = -1e30f;
+    l[i] = 0.f;
+#pragma unroll
+    for (int v = 0; v < VPL; ++v) acc[i][v] = 0.f;
+  }
+  float* my_p = p_s + w * HM * 64;
+  int64_t* my_off = off_s + w * 64;
+
+  for (int tile = first + 64 * w; tile <= last; tile += 256) {
+    const int j = tile + lane;
+    const bool valid = j <= last;
+    const int jc = min(j, last);   // a key that is not there: the last one's row in its place
+    const int64_t at = ((int64_t)bt[jc / a.page_size] * a.Hkv + g) * a.page_size + jc % a.page_size;
+    typedef unsigned int uint4v __attribute__((ext_vector_type(4)));
+    const uint4v* kr = (const uint4v*)(kpool + at * kd);
+    float dots[HM];
+#pragma unroll
+    for (int i = 0; i < HM; ++i) dots[i] = 0.f;
+#pragma unroll
+    for (int mp = 0; mp < 2; ++mp)
+      for (int d8 = 0; d8 < dim / 8; ++d8) {
+        const uint4v kk = stream_load(kr + mp * (dim / 8) + d8);
+        float kf[8];
+        kf[0] = __uint_as_float(kk.x << 16); kf[1] = __uint_as_float(kk.x & 0xffff0000u);
+        kf[2] = __uint_as_float(kk.y << 16); kf[3] = __uint_as_float(kk.y & 0xffff0000u);
+        kf[4] = __uint_as_float(kk.z << 16); kf[5] = __uint_as_float(kk.z & 0xffff0000u);
+        kf[6] = __uint_as_float(kk.w << 16); kf[7] = __uint_as_float(kk.w & 0xffff0000u);
+#pragma unroll
+        for (int hb = 0; hb < HB; ++hb) {
+          const float4 qa = *(const float4*)(q_s + hb * kd + mp * dim + d8 * 8);
+          const float4 qb = *(const float4*)(q_s + hb * kd + mp * dim + d8 * 8 + 4);
+          float s = dots[2 * hb + mp];
+          s = fmaf(qa.x, kf[0], s); s = fmaf(qa.y, kf[1], s); s = fmaf(qa.z, kf[2], s); s = fmaf(qa.w, kf[3], s);
+          s = fmaf(qb.x, kf[4], s); s = fmaf(qb.y, kf[5], s); s = fmaf(qb.z, kf[6], s); s = fmaf(qb.w, kf[7], s);
+          dots[2 * hb + mp] = s;
+        }
+      }
+    float alpha[HM];
+#pragma unroll
+    for (int i = 0; i < HM; ++i) {
+      float s = dots[i] * qscale;
+      if (a.cap > 0.f) s = a.cap * tanhf(s / a.cap);
+      if (!valid) s = -INFINITY;
+      const float m_new = fmaxf(m[i], wave_max(s));
+      const float p = valid ? expf(s - m_new) : 0.f;
+      alpha[i] = expf(m[i] - m_new);
+      l[i] = l[i] * alpha[i] + wave_sum(p);
+      m[i] = m_new;
+      my_p[i * 64 + lane] = p;
+    }
+    my_off[lane] = at * vdim;
+    __builtin_amdgcn_wave_barrier();   // the wave's own writes above are read below, in order
+    const int n_keys = min(64, last - tile + 1);
+#pragma unroll
+    for (int i = 0; i < HM; ++i)
+#pragma unroll
+      for (int v = 0; v < VPL; ++v) acc[i][v] *= alpha[i];
+    for (int jj = 0; jj < n_keys; ++jj) {
+      const bf16* vr = vpool + my_off[jj];
+      float val[VPL];
+#pragma unroll
+      for (int v = 0; v < VPL; ++v) val[v] = lane + 64 * v < vdim ? to_f32(vr[lane + 64 * v]) : 0.f;
+#pragma unroll
+      for (int i = 0; i < HM; ++i) {
+        const float p = my_p[i * 64 + jj];
+#pragma unroll
+        for (int v = 0; v < VPL; ++v) acc[i][v] = fmaf(p, val[v], acc[i][v]);
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+  // the four waves' sums put together: wave hb finishes head hb
+  if (lane == 0)
+    for (int i = 0; i < HM; ++i) {
+      ml_s[(w * HM + i) * 2] = m[i];
+      ml_s[(w * HM + i) * 2 + 1] = l[i];
+    }
+#pragma unroll
+  for (int i = 0; i < HM; ++i)
+#pragma unroll
+    for (int v = 0; v < VPL; ++v) acc_s[((w * HM + i) * VPL + v) * 64 + lane] = acc[i][v];
+  __syncthreads();
+  if (w >= HB) return;
+  float fm[2], fl[2], facc[2][kMaxVPerLane];
+#pragma unroll
+  for (int mp = 0; mp < 2; ++mp) {
+    const int i = 2 * w + mp;
+    float mm = -1e30f;
+    for (int x = 0; x < 4; ++x) mm = fmaxf(mm, ml_s[(x * HM + i) * 2]);
+    float ll = 0.f;
+#pragma unroll
+    for (int v = 0; v < kMaxVPerLane; ++v) facc[mp][v] = 0.f;
+    for (int x = 0; x < 4; ++x) {
+      const float f = expf(ml_s[(x * HM + i) * 2] - mm);
+      ll += f * ml_s[(x * HM + i) * 2 + 1];
+#pragma unroll
+      for (int v = 0; v < VPL; ++v) facc[mp][v] = fmaf(f, acc_s[((x * HM + i) * VPL + v) * 64 + lane], facc[mp][v]);
+    }
+    fm[mp] = mm;
+    fl[mp] = ll;
+  }
+  const int h = h0 + w;
+  if (n_chunks == 1) {
+    diff_finish<bf16>(a, facc[0], facc[1], fl[0], fl[1], (bf16*)a.out + ((int64_t)t * a.Hq + h) * vdim, lane);
+    return;
+  }
+  float* part = a.workspace + (((int64_t)t * a.Hq + h) * n_chunks + c) * (4 + 2 * vdim);
+  if (lane == 0) {
+    part[0] = fm[0];
+    part[1] = fl[0];
+    part[2] = fm[1];
+    part[3] = fl[1];
+  }
+#pragma unroll
+  for (int v = 0; v < VPL; ++v) {
+    const int d = lane + 64 * v;
+    if (d < vdim) {
+      part[4 + d] = facc[0][v];
+      part[4 + vdim + d] = facc[1][v];
+    }
+  }
+}
+
+static bool diff_rows_takes(const DiffAttnArgs& a) {
+  return a.dtype == kBF16 && a.max_qlen == 1 && !a.force_plain && a.dim % 8 == 0 && a.vdim <= 256 &&
+         a.q_stride % 8 == 0;
+}
+
+static int diff_rows_heads(const DiffAttnArgs& a) {
+  const int hpg = a.Hq / a.Hkv;
+  return hpg % 4 == 0 ? 4 : (hpg % 2 == 0 ? 2 : 1);
+}
+
+template <int HB>
+static int launch_rows(const DiffAttnArgs& a, int chunk, int n_chunks, hipStream_t stream) {
+  const int vpl = (a.vdim + 63) / 64;
+  const size_t lds = (size_t)(HB * 2 * a.dim + 4 * 2 * HB * 64 + 4 * 2 * HB * 2 + 4 * 2 * HB * vpl * 64) * sizeof(float) +
+                     4 * 64 * sizeof(int64_t);
+  dim3 grid(a.T, a.Hkv * (a.Hq / a.Hkv / HB), n_chunks);
+  switch (vpl) {
+    case 1: diff_attention_rows_kernel<HB, 1><<<grid, 256, lds, stream>>>(a, chunk, n_chunks); break;
+    case 2: diff_attention_rows_kernel<HB, 2><<<grid, 256, lds, stream>>>(a, chunk, n_chunks); break;
+    case 3: diff_attention_rows_kernel<HB, 3><<<grid, 256, lds, stream>>>(a, chunk, n_chunks); break;
+    default: diff_attention_rows_kernel<HB, 4><<<grid, 256, lds, stream>>>(a, chunk, n_chunks); break;
+  }
+  NINFER_LAUNCH_CHECK();
+  if (n_chunks > 1) {
+    diff_attention_merge_kernel<bf16><<<dim3(a.T, a.Hq), 64, 0, stream>>>(a, n_chunks);
+    NINFER_LAUNCH_CHECK();
+  }
+  return 0;
+}
+
+static int diff_attention_rows(const DiffAttnArgs& a, int chunk, int n_chunks, hipStream_t stream) {
+  switch (diff_rows_heads(a)) {
+    case 4: return launch_rows<4>(a, chunk, n_chunks, stream);
+    case 2: return launch_rows<2>(a, chunk, n_chunks, stream);
+    default: return launch_rows<1>(a, chunk, n_chunks, stream);
+  }
+}
+
 int diff_attention_plain(const DiffAttnArgs& a, int chunk, int n_chunks, hipStream_t stream) {
   const size_t lds = (2 * a.dim + 128 + 2) * sizeof(float) + 64 * sizeof(int64_t);
   dim3 grid(a.T, a.Hq, n_chunks);
@@ -216,10 +417,18 @@ static void diff_chunks(const DiffAttnArgs& a, int* chunk, int* n_chunks) {
   *chunk = 0;
   *n_chunks = 1;
   if (a.dtype != kBF16 || a.max_qlen != 1 || a.force_plain) return;
-  const int waves = a.T * a.Hq;
-  const int want = (8 * device_cu_count() + waves - 1) / waves;   // eight waves a CU
-  int per = (a.max_kv_len + want - 1) / want;
-  per = ((per < 256 ? 256 : per) + 63) / 64 * 64;
+  int per;
+  if (diff_rows_takes(a)) {
+    // blocks of four waves, each wave a tile of 64 keys at a time: two blocks a CU
+    const int blocks = a.T * (a.Hq / diff_rows_heads(a));
+    const int want = (2 * device_cu_count() + blocks - 1) / blocks;
+    per = (a.max_kv_len + want - 1) / want;
+  } else {
+    const int waves = a.T * a.Hq;
+    const int want = (8 * device_cu_count() + waves - 1) / waves;   // eight waves a CU
+    per = (a.max_kv_len + want - 1) / want;
+  }
+  per = ((per < 256 ? 256 : per) + 255) / 256 * 256;
   const int n = (a.max_kv_len + per - 1) / per;
   if (n > 1) {
     *chunk = per;
@@ -270,5 +479,6 @@ extern "C" int ninfer_diff_attention(const DiffAttnArgs* a, hipStream_t stream) 
   if (n > 1)
     NINFER_REQUIRE(a->workspace && a->workspace_floats >= (int64_t)a->T * a->Hq * n * (4 + 2 * a->vdim),
                    "diff_attention: the workspace is too small for %d chunks", n);
+  if (diff_rows_takes(*a)) return diff_attention_rows(*a, chunk, n, stream);
   return diff_attention_plain(*a, chunk, n, stream);
 }

@@ -8,8 +8,15 @@ namespace ninfer {
 
 // A gated epilogue forms act(x Wg^T) * (x Wu^T) from the two halves of W's rows; the
 // activation is SiLU (SwiGLU) or the tanh form of GELU (GeGLU).
-enum Epilogue : int { kEpilogueNone = 0, kEpilogueSwiGLU = 1, kEpilogueGeGLU = 2 };
+// kEpilogueReluSq is not gated: every output (after its bias) becomes max(., 0)^2.
+enum Epilogue : int { kEpilogueNone = 0, kEpilogueSwiGLU = 1, kEpilogueGeGLU = 2, kEpilogueReluSq = 3 };
 inline bool epilogue_gated(int e) { return e == kEpilogueSwiGLU || e == kEpilogueGeGLU; }
+// What an ungated epilogue makes of an output.
+__device__ __forceinline__ float ungated_output(float v, bool relu_sq) {
+  if (!relu_sq) return v;
+  const float r = fmaxf(v, 0.f);
+  return r * r;
+}
 
 // Both activations are g * sigmoid(z): z = g for SiLU; for GELU's tanh form,
 // 0.5 g (1 + tanh(c (g + 0.044715 g^3))) with c = sqrt(2 / pi), z = 2 c (g + 0.044715 g^3).

@@ -111,8 +111,9 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(GemmArgs a) {
         float g = v + (a.bias ? a.bias[n] : 0.f);
         const float u = accu[i][j] + (a.bias ? a.bias[a.N + n] : 0.f);
         v = g / (1.f + expf(-gate_logit(g, a.epilogue == kEpilogueGeGLU))) * u;
-      } else if (a.bias) {
-        v += a.bias[n];
+      } else {
+        if (a.bias) v += a.bias[n];
+        v = ungated_output(v, a.epilogue == kEpilogueReluSq);
       }
       C[c_row * a.ldc + n] = from_f32<TC>(v);
     }
@@ -143,7 +144,7 @@ int gemm_check(const GemmArgs& a) {
   NINFER_REQUIRE(a.groups >= 1, "gemm: groups=%d must be >= 1", a.groups);
   NINFER_REQUIRE(a.offsets || a.groups == 1, "gemm: %d groups without offsets", a.groups);
   NINFER_REQUIRE(!a.a_index || a.a_div >= 1, "gemm: a_div=%d must be >= 1", a.a_div);
-  NINFER_REQUIRE(a.epilogue == kEpilogueNone || epilogue_gated(a.epilogue),
+  NINFER_REQUIRE(a.epilogue == kEpilogueNone || epilogue_gated(a.epilogue) || a.epilogue == kEpilogueReluSq,
                  "gemm: unknown epilogue %d", a.epilogue);
   NINFER_REQUIRE(!(epilogue_gated(a.epilogue) && a.bias && a.offsets),
                  "gemm: a grouped product with a gated epilogue takes no bias");

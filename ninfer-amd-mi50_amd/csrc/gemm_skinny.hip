@@ -238,8 +238,9 @@ __device__ __forceinline__ void skinny_block(const GemmArgs& a, int rows_arg, in
             u += a.bias[a.N + col];
           }
           v = v / (1.f + __expf(-gate_logit(v, a.epilogue == kEpilogueGeGLU))) * u;
-        } else if (a.bias) {
-          v += a.bias[col];
+        } else {
+          if (a.bias) v += a.bias[col];
+          v = ungated_output(v, a.epilogue == kEpilogueReluSq);
         }
         ((TC*)a.C)[c_row * a.ldc + col] = from_f32<TC>(v);
       }

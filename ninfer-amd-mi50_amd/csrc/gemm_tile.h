@@ -112,6 +112,7 @@ __device__ inline void write_accumulators(const GemmArgs& a, const f32x16 (&acc)
   // four features side by side go out in one store when every such group is whole and aligned
   const bool whole_quads = N % 4 == 0 && a.ldc % 4 == 0 && ((uintptr_t)a.C & 15) == 0;
   const bool gelu = a.epilogue == kEpilogueGeGLU;
+  const bool relu_sq = a.epilogue == kEpilogueReluSq;
 #pragma unroll
   for (int jj = 0; jj < FJ; ++jj) {
     const int r_tile = row_of(tok0 + 32 * jj + lr);
@@ -154,6 +155,7 @@ __device__ inline void write_accumulators(const GemmArgs& a, const f32x16 (&acc)
           for (int r = 0; r < 4; ++r) {
             v[r] = acc[i][jj][4 * q + r];
             if (a.bias && f0 + r < N) v[r] += a.bias[f0 + r];
+            v[r] = ungated_output(v[r], relu_sq);
           }
           if (whole_quads) {   // N % 4 == 0: the four features are in or out together
             if (f0 < N) store_quad(crow + f0, v);
@@ -187,6 +189,7 @@ __device__ inline void write_accumulators_staged(const GemmArgs& a, const f32x16
   const int lane = threadIdx.x & 63, lr = lane & 31, lk = lane >> 5;
   const int N = a.N;
   const bool gelu = a.epilogue == kEpilogueGeGLU;
+  const bool relu_sq = a.epilogue == kEpilogueReluSq;
 #pragma unroll
   for (int jj = 0; jj < FJ; ++jj) {
     const int tok = 32 * jj + lr;
@@ -219,7 +222,7 @@ __device__ inline void write_accumulators_staged(const GemmArgs& a, const f32x16
             for (int r = 0; r < 4; ++r) b[r] = a.bias[f + r];
           }
 #pragma unroll
-          for (int r = 0; r < 4; ++r) val[r] = (__bf16)(acc[i][jj][4 * q + r] + b[r]);
+          for (int r = 0; r < 4; ++r) val[r] = (__bf16)ungated_output(acc[i][jj][4 * q + r] + b[r], relu_sq);
         }
         const int v = 4 * i + q;
         *(bf16x4*)(stage + tok * RB + ((v ^ (tok & (U - 1))) << 4) + 8 * lk) = val;

@@ -61,6 +61,8 @@ ROUTE_MANY_MIN_ROWS = 2048
 _SCORES = {"softmax": 0, "sigmoid": 1}
 # activations of a gated product, by the names config.json gives them -> the library's epilogue
 GATE_ACTS = {"silu": 1, "gelu_pytorch_tanh": 2}
+# ... and of a plain product: none, or the square of relu on every output
+UNGATED_ACTS = {None: 0, "relu2": 3}
 
 
 class _AttnArgs(ctypes.Structure):
@@ -631,11 +633,8 @@ class HipOps:
     def linear(self, x, w, out, bias=None, act=None):
         """out = x w^T (+ bias); out may be 32-bit whatever the inputs are. `act` 'relu2': the
         square of relu on every element of out."""
-        if act is not None:
-            _need(act == "relu2", f"linear: activation {act!r} is not 'relu2'")
-            self.linear(x, w, out, bias)
-            self.relu_square(out)
-            return
+        # (an activation runs in the product's epilogue, on the kernels here at every row count)
+        _need(act in UNGATED_ACTS, f"linear: activation {act!r} is not one of {sorted(map(str, UNGATED_ACTS))}")
         _dev(x, "x", dims=2)
         _dev(w, "w", x.dtype, 2)
         _dev(out, "out", dims=2)
@@ -645,14 +644,15 @@ class HipOps:
         if bias is not None:
             _dev(bias, "bias", torch.float32, 1)
             _need(bias.shape[0] == w.shape[0], "linear: bias has the wrong size")
-        if self._use_library(x, out, w) and bias is None and not (
+        if act is None and self._use_library(x, out, w) and bias is None and not (
                 x.shape[0] <= self.side_own_max_rows
                 and w.numel() * w.element_size() <= self.side_own_max_bytes and self._on_side()):
             if x.shape[0] > self.split_max_rows or not self._gemm(
                     x, w, out, m=x.shape[0], n=w.shape[0], k=x.shape[1], only_if_split=True):
                 torch.matmul(x, w.t(), out=out)
             return
-        self._gemm(x, w, out, m=x.shape[0], n=w.shape[0], k=x.shape[1], bias=bias)
+        self._gemm(x, w, out, m=x.shape[0], n=w.shape[0], k=x.shape[1], bias=bias,
+                   epilogue=UNGATED_ACTS[act])
 
     def _use_library(self, x, out, w) -> bool:
         """Plain dense products of many bf16 rows go to the vendor library, as

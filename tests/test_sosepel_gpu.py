@@ -163,6 +163,26 @@ def test_small_row_kernels(ops):
     torch.testing.assert_close(y.cpu().double(), 7.5 * torch.tanh(x.double() / 7.5), atol=1e-5, rtol=1e-5)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows", [1, 5, 20, 40, 70, 300])
+def test_product_with_the_square_of_relu(ops, dtype, rows):
+    """The activation runs in the product's epilogue, whichever kernel the row count picks."""
+    torch.manual_seed(rows)
+    for k, n in ((72, 100), (256, 512), (2048, 1408)):
+        x, w = (torch.randn(rows, k) * 0.5).to(dtype), (torch.randn(n, k) * 0.1).to(dtype)
+        want = torch.relu(x.double() @ w.double().T) ** 2
+        out = torch.empty(rows, n, dtype=dtype, device=DEV)
+        ops.linear(x.to(DEV), w.to(DEV), out, act="relu2")
+        assert rel_err(out, want) < (1e-5 if dtype == torch.float32 else 6e-3)
+        with ops.tuned(force_kernel=0):
+            ops.force_generic = True
+            try:
+                ops.linear(x.to(DEV), w.to(DEV), out, act="relu2")
+            finally:
+                ops.force_generic = False
+        assert rel_err(out, want) < (1e-5 if dtype == torch.float32 else 6e-3)
+
+
 @pytest.mark.parametrize("experts,top,count,keep", [(6, 3, 3, 2), (16, 4, 2, 1), (9, 2, 3, 1), (4, 2, 4, 3),
                                                      (128, 6, 8, 3), (12, 5, 1, 1), (70, 2, 7, 2)])
 def test_choice_limited_to_groups_by_their_two_best(ops, experts, top, count, keep):
