@@ -45,5 +45,11 @@ struct DiffAttnArgs {
 int diff_attention_plain(const DiffAttnArgs& a, int chunk, int n_chunks, hipStream_t stream);
 bool diff_attention_tiles_takes(const DiffAttnArgs& a);
 int diff_attention_tiles(const DiffAttnArgs& a, hipStream_t stream);
+// single rows with the heads of a kv head as the tile's rows: chunks, then the merge
+bool diff_attention_heads_takes(const DiffAttnArgs& a);
+void diff_attention_heads_plan(const DiffAttnArgs& a, int* chunk, int* n_chunks);
+int diff_attention_heads(const DiffAttnArgs& a, int chunk, int n_chunks, hipStream_t stream);
+// the records {m1, l1, m2, l2, acc1[vdim], acc2[vdim]} of every row and head put together
+int diff_attention_merge(const DiffAttnArgs& a, int n_records, hipStream_t stream);
 
 }  // namespace ninfer

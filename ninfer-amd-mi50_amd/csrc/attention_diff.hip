@@ -412,6 +412,13 @@ int diff_attention_plain(const DiffAttnArgs& a, int chunk, int n_chunks, hipStre
   return 0;
 }
 
+int diff_attention_merge(const DiffAttnArgs& a, int n_records, hipStream_t stream) {
+  if (a.dtype == kF32) diff_attention_merge_kernel<float><<<dim3(a.T, a.Hq), 64, 0, stream>>>(a, n_records);
+  else diff_attention_merge_kernel<bf16><<<dim3(a.T, a.Hq), 64, 0, stream>>>(a, n_records);
+  NINFER_LAUNCH_CHECK();
+  return 0;
+}
+
 // Single rows (a decode step): how the contexts are cut so that the launch fills the GPU.
 static void diff_chunks(const DiffAttnArgs& a, int* chunk, int* n_chunks) {
   *chunk = 0;
@@ -464,6 +471,10 @@ extern "C" int ninfer_diff_kv_write(const DiffAttnArgs* a, hipStream_t stream) {
 
 extern "C" long long ninfer_diff_attention_workspace_floats(const DiffAttnArgs* a) {
   int chunk, n;
+  if (!a->force_plain && diff_attention_heads_takes(*a)) {
+    diff_attention_heads_plan(*a, &chunk, &n);
+    return (long long)a->T * a->Hq * 2 * n * (4 + 2 * a->vdim);
+  }
   diff_chunks(*a, &chunk, &n);
   return n > 1 ? (long long)a->T * a->Hq * n * (4 + 2 * a->vdim) : 0;
 }
@@ -475,6 +486,10 @@ extern "C" int ninfer_diff_attention(const DiffAttnArgs* a, hipStream_t stream) 
   if (a->max_qlen > 1 && !a->force_plain && diff_attention_tiles_takes(*a))
     return diff_attention_tiles(*a, stream);
   int chunk, n;
+  if (!a->force_plain && diff_attention_heads_takes(*a)) {
+    diff_attention_heads_plan(*a, &chunk, &n);
+    return diff_attention_heads(*a, chunk, n, stream);
+  }
   diff_chunks(*a, &chunk, &n);
   if (n > 1)
     NINFER_REQUIRE(a->workspace && a->workspace_floats >= (int64_t)a->T * a->Hq * n * (4 + 2 * a->vdim),

@@ -275,7 +275,8 @@ def _cut(n, sizes, tail):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("heads,kv_heads,dim,vdim,ps", [(6, 3, 12, 20, 8), (4, 1, 32, 64, 16), (2, 2, 16, 32, 4),
                                                         (4, 2, 64, 128, 16), (6, 2, 40, 72, 32),
-                                                        (1, 1, 128, 8, 16), (8, 2, 24, 96, 2)])
+                                                        (1, 1, 128, 8, 16), (8, 2, 24, 96, 2),
+                                                        (2, 1, 136, 160, 8), (4, 2, 16, 40, 12), (40, 1, 8, 16, 16)])
 def test_differential_attention_in_portions(ops, dtype, heads, kv_heads, dim, vdim, ps):
     """Three requests of unequal length side by side: portions that end before, at and after
     the borders of pages and of the kernels' tiles of 64 keys, down to two rows, then rows one
