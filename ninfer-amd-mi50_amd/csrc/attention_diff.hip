@@ -164,34 +164,87 @@ __global__ __launch_bounds__(64) void diff_attention_plain_kernel(DiffAttnArgs a
   }
 }
 
-// The chunks of a row and head put together, in the chunks' order (a chunk that starts
-// beyond the row's position holds l = 0 and counts for nothing).
+// The records of a row and head put together by a block of four waves (a record whose l is 0
+// counts for nothing: a chunk that starts beyond the row's position, a wave that met no key).
+// The threads first take a record each: the largest m of each map, then every record's weight
+// exp(m - M) into LDS and the sum of the weighted l; then wave w adds up the weighted records
+// w, w + 4, ... over its lanes' value columns, and the first wave adds the four sums and
+// finishes the head.
 template <typename T>
-__global__ __launch_bounds__(64) void diff_attention_merge_kernel(DiffAttnArgs a, int n_chunks) {
-  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+__global__ __launch_bounds__(256) void diff_attention_merge_kernel(DiffAttnArgs a, int n_records) {
+  extern __shared__ float w_s[];          // [2][n_records], then 16 for reductions, then [4][2][vdim]
+  float* red = w_s + 2 * n_records;
+  float* acc_s = red + 16;
+  const int t = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int stride = 4 + 2 * a.vdim;
-  const float* part = a.workspace + ((int64_t)t * a.Hq + h) * n_chunks * stride;
+  const float* part = a.workspace + ((int64_t)t * a.Hq + h) * n_records * stride;
   float m1 = -INFINITY, m2 = -INFINITY;
-  for (int c = 0; c < n_chunks; ++c) {
-    if (part[c * stride + 1] > 0.f) m1 = fmaxf(m1, part[c * stride]);
-    if (part[c * stride + 3] > 0.f) m2 = fmaxf(m2, part[c * stride + 2]);
+  for (int c = tid; c < n_records; c += 256) {
+    const float* r = part + (int64_t)c * stride;
+    if (r[1] > 0.f) m1 = fmaxf(m1, r[0]);
+    if (r[3] > 0.f) m2 = fmaxf(m2, r[2]);
   }
+  m1 = wave_max(m1);
+  m2 = wave_max(m2);
+  if (lane == 0) {
+    red[w] = m1;
+    red[4 + w] = m2;
+  }
+  __syncthreads();
+  m1 = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  m2 = fmaxf(fmaxf(red[4], red[5]), fmaxf(red[6], red[7]));
   float l1 = 0.f, l2 = 0.f;
+  for (int c = tid; c < n_records; c += 256) {
+    const float* r = part + (int64_t)c * stride;
+    const float w1 = r[1] > 0.f ? expf(r[0] - m1) : 0.f, w2 = r[3] > 0.f ? expf(r[2] - m2) : 0.f;
+    w_s[c] = w1;
+    w_s[n_records + c] = w2;
+    l1 += w1 > 0.f ? w1 * r[1] : 0.f;
+    l2 += w2 > 0.f ? w2 * r[3] : 0.f;
+  }
+  l1 = wave_sum(l1);
+  l2 = wave_sum(l2);
+  if (lane == 0) {
+    red[8 + w] = l1;
+    red[12 + w] = l2;
+  }
+  __syncthreads();
+  l1 = (red[8] + red[9]) + (red[10] + red[11]);
+  l2 = (red[12] + red[13]) + (red[14] + red[15]);
   float acc1[kMaxVPerLane], acc2[kMaxVPerLane];
 #pragma unroll
   for (int i = 0; i < kMaxVPerLane; ++i) acc1[i] = acc2[i] = 0.f;
-  for (int c = 0; c < n_chunks; ++c) {
-    const float* p = part + c * stride;
-    const float w1 = p[1] > 0.f ? expf(p[0] - m1) : 0.f, w2 = p[3] > 0.f ? expf(p[2] - m2) : 0.f;
-    l1 += w1 * p[1];
-    l2 += w2 * p[3];
+#pragma unroll 4
+  for (int c = w; c < n_records; c += 4) {
+    const float* p = part + (int64_t)c * stride + 4;
+    const float w1 = w_s[c], w2 = w_s[n_records + c];
 #pragma unroll
     for (int i = 0; i < kMaxVPerLane; ++i) {
       const int d = lane + i * 64;
       if (d < a.vdim) {
-        if (w1 > 0.f) acc1[i] = fmaf(w1, p[4 + d], acc1[i]);
-        if (w2 > 0.f) acc2[i] = fmaf(w2, p[4 + a.vdim + d], acc2[i]);
+        // (a record that counts for nothing may hold anything: it does not enter the sum)
+        const float x1 = p[d], x2 = p[a.vdim + d];
+        acc1[i] += w1 > 0.f ? w1 * x1 : 0.f;
+        acc2[i] += w2 > 0.f ? w2 * x2 : 0.f;
       }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < kMaxVPerLane; ++i) {
+    const int d = lane + i * 64;
+    if (d < a.vdim) {
+      acc_s[(w * 2) * a.vdim + d] = acc1[i];
+      acc_s[(w * 2 + 1) * a.vdim + d] = acc2[i];
+    }
+  }
+  __syncthreads();
+  if (w != 0) return;
+#pragma unroll
+  for (int i = 0; i < kMaxVPerLane; ++i) {
+    const int d = lane + i * 64;
+    if (d < a.vdim) {
+      acc1[i] = (acc_s[d] + acc_s[2 * a.vdim + d]) + (acc_s[4 * a.vdim + d] + acc_s[6 * a.vdim + d]);
+      acc2[i] = (acc_s[a.vdim + d] + acc_s[3 * a.vdim + d]) + (acc_s[5 * a.vdim + d] + acc_s[7 * a.vdim + d]);
     }
   }
   diff_finish<T>(a, acc1, acc2, l1, l2, (T*)a.out + ((int64_t)t * a.Hq + h) * a.vdim, lane);
@@ -384,7 +437,7 @@ static int launch_rows(const DiffAttnArgs& a, int chunk, int n_chunks, hipStream
   }
   NINFER_LAUNCH_CHECK();
   if (n_chunks > 1) {
-    diff_attention_merge_kernel<bf16><<<dim3(a.T, a.Hq), 64, 0, stream>>>(a, n_chunks);
+    diff_attention_merge_kernel<bf16><<<dim3(a.T, a.Hq), 256, (2 * n_chunks + 16 + 8 * a.vdim) * sizeof(float), stream>>>(a, n_chunks);
     NINFER_LAUNCH_CHECK();
   }
   return 0;
@@ -403,18 +456,18 @@ int diff_attention_plain(const DiffAttnArgs& a, int chunk, int n_chunks, hipStre
   dim3 grid(a.T, a.Hq, n_chunks);
   if (a.dtype == kF32) {
     diff_attention_plain_kernel<float><<<grid, 64, lds, stream>>>(a, chunk, n_chunks);
-    if (n_chunks > 1) diff_attention_merge_kernel<float><<<dim3(a.T, a.Hq), 64, 0, stream>>>(a, n_chunks);
+    if (n_chunks > 1) diff_attention_merge_kernel<float><<<dim3(a.T, a.Hq), 256, (2 * n_chunks + 16 + 8 * a.vdim) * sizeof(float), stream>>>(a, n_chunks);
   } else {
     diff_attention_plain_kernel<bf16><<<grid, 64, lds, stream>>>(a, chunk, n_chunks);
-    if (n_chunks > 1) diff_attention_merge_kernel<bf16><<<dim3(a.T, a.Hq), 64, 0, stream>>>(a, n_chunks);
+    if (n_chunks > 1) diff_attention_merge_kernel<bf16><<<dim3(a.T, a.Hq), 256, (2 * n_chunks + 16 + 8 * a.vdim) * sizeof(float), stream>>>(a, n_chunks);
   }
   NINFER_LAUNCH_CHECK();
   return 0;
 }
 
 int diff_attention_merge(const DiffAttnArgs& a, int n_records, hipStream_t stream) {
-  if (a.dtype == kF32) diff_attention_merge_kernel<float><<<dim3(a.T, a.Hq), 64, 0, stream>>>(a, n_records);
-  else diff_attention_merge_kernel<bf16><<<dim3(a.T, a.Hq), 64, 0, stream>>>(a, n_records);
+  if (a.dtype == kF32) diff_attention_merge_kernel<float><<<dim3(a.T, a.Hq), 256, (2 * n_records + 16 + 8 * a.vdim) * sizeof(float), stream>>>(a, n_records);
+  else diff_attention_merge_kernel<bf16><<<dim3(a.T, a.Hq), 256, (2 * n_records + 16 + 8 * a.vdim) * sizeof(float), stream>>>(a, n_records);
   NINFER_LAUNCH_CHECK();
   return 0;
 }

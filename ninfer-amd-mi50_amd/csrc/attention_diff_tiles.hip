@@ -1,8 +1,10 @@
 // Differential attention for prompt portions on the matrix cores (bf16 rows and cache).
 //
-// A block of four waves owns one kv head and a tile of rows of one request: every wave 32
-// rows of one query head (HB query heads of the kv head side by side, 4 / HB groups of 32
-// rows), so that all waves meet the same keys and values. These are walked in tiles of 64
+// A block of four waves owns one kv head and a tile of rows of one request: a pair of waves
+// owns 32 rows of one query head, one wave for each map (HB = 2 or 1 query heads of the kv
+// head side by side, 2 / HB groups of 32 rows), so that all waves meet the same keys and
+// values and a wave's registers hold one map's output only (two blocks fit a CU, and one
+// wave's softmax arithmetic runs beside another's matrix products). These are walked in tiles of 64
 // keys aligned to absolute positions: global memory -> registers (one tile ahead) -> LDS, two
 // buffers, one barrier per tile. A key row lies in LDS as [map 1 | map 2], each padded with
 // zeros to DP = 16 KS numbers; a value row padded to VP = 32 DB.
@@ -14,9 +16,10 @@
 // probabilities, rounded to bf16 in place, are the B operand of
 //   O^T[value column][row] += V^T P^T   (A = V^T: the transposing LDS read hands a lane four
 //                                        consecutive keys of one value column)
-// with the contraction index numbered as the lanes hold it. Both maps read the same value
-// fragments. At the end o = O1 / l1 - lambda O2 / l2, the head's norm over its value columns,
-// the factor, the store.
+// with the contraction index numbered as the lanes hold it. At the end the wave of map 2
+// hands lambda O2 / l2 to its partner through LDS (the tiles' buffers, lane by lane: both hold
+// the same places), which forms o = O1 / l1 - lambda O2 / l2, the head's norm over its value
+// columns, the factor, and stores.
 // Keys that do not exist (beyond the tile's last row) load the last row's key in their place:
 // they are masked, and their values must be finite since 0 x NaN is not 0.
 #include "attention_diff.h"
@@ -33,7 +36,7 @@ typedef __attribute__((address_space(3))) short4v lds_short4;
 constexpr float kLog2e = 1.44269504088896f;
 
 template <int KS, int DB>
-__global__ __launch_bounds__(256) void diff_attention_tiles_kernel(DiffAttnArgs a, int HB) {
+__global__ __launch_bounds__(256, 2) void diff_attention_tiles_kernel(DiffAttnArgs a, int HB) {
   constexpr int DP = 16 * KS, KROW = 2 * DP + 8, VP = 32 * DB, VROW = VP + 8;
   constexpr int TILE = 64 * KROW + 64 * VROW;   // elements of one buffer
   extern __shared__ __attribute__((aligned(16))) unsigned short lds[];
@@ -41,15 +44,16 @@ __global__ __launch_bounds__(256) void diff_attention_tiles_kernel(DiffAttnArgs 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int c = lane & 31, hi = lane >> 5;
   const int hpg = a.Hq / a.Hkv;
-  const int RT = 32 * (4 / HB);
+  const int mp = wave & 1, unit = wave >> 1;   // the wave's map; its pair's place in the block
+  const int RT = 32 * (2 / HB);
   const int g = blockIdx.y / (hpg / HB);
-  const int h = g * hpg + (blockIdx.y % (hpg / HB)) * HB + wave % HB;
-  const int rs = wave / HB;
+  const int h = g * hpg + (blockIdx.y % (hpg / HB)) * HB + unit % HB;
+  const int rs = unit / HB;
 
   // which request and which of its row tiles
   int seq = -1, row0 = 0, n_rows = 0;
   {
-    int idx = blockIdx.x;
+    int idx = gridDim.x - 1 - blockIdx.x;   // the last row tiles of a request walk the most keys: first
     for (int s = 0; s < a.S; ++s) {
       const int b = a.seq_row_start[s], e = a.seq_row_start[s + 1];
       const int nt = (e - b + RT - 1) / RT;
@@ -123,25 +127,23 @@ __global__ __launch_bounds__(256) void diff_attention_tiles_kernel(DiffAttnArgs 
       if (v_ok[i]) *(u32x4*)(vs + v_key[i] * VROW + v_src[i]) = vreg[i];                          \
   }
 
-  // this lane's queries (B operand): row c of the wave, dims 16 ks + 8 hi .. + 7 of each map
+  // this lane's queries (B operand): row c of the wave, dims 16 ks + 8 hi .. + 7 of its map
   const bool wave_live = rs * 32 < n_rows;
   const int q_local = rs * 32 + c;
   const bool q_valid = q_local < n_rows;
   const int q_pos = pos_first + q_local;
   const int wave_last = pos_first + min(rs * 32 + 31, n_rows - 1);
-  bf16x8 qf[2][KS];
+  bf16x8 qf[KS];
   {
     const unsigned short* qr = (const unsigned short*)a.qkv +
-                               (int64_t)(row0 + (q_valid ? q_local : 0)) * a.q_stride + h * kd;
+                               (int64_t)(row0 + (q_valid ? q_local : 0)) * a.q_stride + h * kd + mp * dim;
 #pragma unroll
-    for (int mp = 0; mp < 2; ++mp)
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const int d = 16 * ks + 8 * hi;
-        u32x4 v = {0u, 0u, 0u, 0u};
-        if (d < dim) v = *(const u32x4*)(qr + mp * dim + d);
-        qf[mp][ks] = __builtin_bit_cast(bf16x8, v);
-      }
+    for (int ks = 0; ks < KS; ++ks) {
+      const int d = 16 * ks + 8 * hi;
+      u32x4 v = {0u, 0u, 0u, 0u};
+      if (d < dim) v = *(const u32x4*)(qr + d);
+      qf[ks] = __builtin_bit_cast(bf16x8, v);
+    }
   }
   // scores in units of log 2: (q . k) qscale, capped, times log2(e)
   const float qscale = a.scale * (a.t_coef == 0.f ? 1.f
@@ -150,14 +152,12 @@ __global__ __launch_bounds__(256) void diff_attention_tiles_kernel(DiffAttnArgs 
   const float pre = capped ? qscale / a.cap * 2.f * kLog2e : qscale * kLog2e;
   const float cap2 = a.cap * kLog2e;
 
-  f32x16 o[2][DB];
+  f32x16 o[DB];
 #pragma unroll
-  for (int mp = 0; mp < 2; ++mp)
+  for (int db = 0; db < DB; ++db)
 #pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) o[mp][db][v] = 0.f;
-  float m[2] = {-1e30f, -1e30f}, l[2] = {0.f, 0.f};
+    for (int v = 0; v < 16; ++v) o[db][v] = 0.f;
+  float m = -1e30f, l = 0.f;
 
   // the transposing read's address of this lane inside a value tile: lane s of a group of 16
   // fetches key s / 4 (+ 4 hi), value columns 16 (group % 2) + 4 (s % 4) .. + 3
@@ -176,65 +176,61 @@ __global__ __launch_bounds__(256) void diff_attention_tiles_kernel(DiffAttnArgs 
     const unsigned short* ks_ = lds + buf * TILE;
     const unsigned short* vs_ = ks_ + 64 * KROW;
     const bool masked = k0 + 63 > pos_first + rs * 32;   // some row of the wave does not see every key
-    bf16x8 pf[2][2][2];
+    f32x16 s[2];
 #pragma unroll
-    for (int mp = 0; mp < 2; ++mp) {
-      f32x16 s[2];
+    for (int kb = 0; kb < 2; ++kb) {
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb) {
+      for (int v = 0; v < 16; ++v) s[kb][v] = 0.f;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) s[kb][v] = 0.f;
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          const bf16x8 kf = *(const bf16x8*)(ks_ + (32 * kb + c) * KROW + mp * DP + 16 * ks + 8 * hi);
-          s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[mp][ks], s[kb], 0, 0, 0);
-        }
+      for (int ks = 0; ks < KS; ++ks) {
+        const bf16x8 kf = *(const bf16x8*)(ks_ + (32 * kb + c) * KROW + mp * DP + 16 * ks + 8 * hi);
+        s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], s[kb], 0, 0, 0);
       }
-      float mx = -__builtin_inff();
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          float x = s[kb][v] * pre;
-          if (capped) {
-            // cap tanh(y) = cap (1 - 2 / (e^(2y) + 1))
-            const float e = __builtin_amdgcn_exp2f(x);
-            x = cap2 * (1.f - 2.f * __builtin_amdgcn_rcpf(e + 1.f));
-          }
-          if (masked) {
-            const int kp = k0 + 32 * kb + 8 * (v >> 2) + 4 * hi + (v & 3);
-            if (kp > q_pos) x = -__builtin_inff();
-          }
-          s[kb][v] = x;
-          mx = fmaxf(mx, x);
-        }
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      const float m_new = fmaxf(m[mp], mx);
-      if (__any(m_new > m[mp])) {
-        const float alpha = __builtin_amdgcn_exp2f(m[mp] - m_new);
-        l[mp] *= alpha;
-#pragma unroll
-        for (int db = 0; db < DB; ++db)
-#pragma unroll
-          for (int v = 0; v < 16; ++v) o[mp][db][v] *= alpha;
-        m[mp] = m_new;
-      }
-      float psum = 0.f;
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-        for (int hh = 0; hh < 2; ++hh)
-#pragma unroll
-          for (int jj = 0; jj < 8; ++jj) {
-            const float p = __builtin_amdgcn_exp2f(s[kb][8 * hh + jj] - m[mp]);
-            psum += p;
-            pf[mp][kb][hh][jj] = (__bf16)p;
-          }
-      l[mp] += psum + __shfl_xor(psum, 32, 64);
     }
+    float mx = -__builtin_inff();
 #pragma unroll
-    for (int db = 0; db < DB; ++db) {
-      bf16x8 vf[2][2];
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        float x = s[kb][v] * pre;
+        if (capped) {
+          // cap tanh(y) = cap (1 - 2 / (e^(2y) + 1))
+          const float e = __builtin_amdgcn_exp2f(x);
+          x = cap2 * (1.f - 2.f * __builtin_amdgcn_rcpf(e + 1.f));
+        }
+        if (masked) {
+          const int kp = k0 + 32 * kb + 8 * (v >> 2) + 4 * hi + (v & 3);
+          if (kp > q_pos) x = -__builtin_inff();
+        }
+        s[kb][v] = x;
+        mx = fmaxf(mx, x);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m, mx);
+    if (__any(m_new > m)) {
+      const float alpha = __builtin_amdgcn_exp2f(m - m_new);
+      l *= alpha;
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) o[db][v] *= alpha;
+      m = m_new;
+    }
+    bf16x8 pf[2][2];
+    float psum = 0.f;
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int hh = 0; hh < 2; ++hh)
+#pragma unroll
+        for (int jj = 0; jj < 8; ++jj) {
+          const float p = __builtin_amdgcn_exp2f(s[kb][8 * hh + jj] - m);
+          psum += p;
+          pf[kb][hh][jj] = (__bf16)p;
+        }
+    l += psum + __shfl_xor(psum, 32, 64);
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
@@ -245,28 +241,33 @@ __global__ __launch_bounds__(256) void diff_attention_tiles_kernel(DiffAttnArgs 
           short8v both;
           both.s0 = lo.x; both.s1 = lo.y; both.s2 = lo.z; both.s3 = lo.w;
           both.s4 = up.x; both.s5 = up.y; both.s6 = up.z; both.s7 = up.w;
-          vf[kb][hh] = __builtin_bit_cast(bf16x8, both);
+          o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, both), pf[kb][hh], o[db], 0, 0, 0);
         }
-#pragma unroll
-      for (int mp = 0; mp < 2; ++mp)
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-          for (int hh = 0; hh < 2; ++hh)
-            o[mp][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[kb][hh], pf[mp][kb][hh], o[mp][db], 0, 0, 0);
-    }
   }
-  if (!wave_live) return;
+  // The pair meets: the wave of map 2 leaves lambda O2 / l2 in LDS, lane by lane (both waves
+  // hold the same rows and columns in the same places), where the tiles were.
+  __syncthreads();   // every wave has read its last tile
+  float* x_s = (float*)lds + unit * (DB * 16 * 64);
+  static_assert(2 * DB * 16 * 64 * 4 <= 2 * TILE * 2, "the pairs' exchange exceeds the tiles' LDS");
+  if (mp == 1 && wave_live) {
+    const float i2 = a.lambda / l;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) x_s[(db * 16 + v) * 64 + lane] = o[db][v] * i2;
+  }
+  __syncthreads();
+  if (mp == 1 || !wave_live) return;
   // o = O1 / l1 - lambda O2 / l2; the norm over the head's value columns; the store. Lane
   // holds, for row c, value columns 32 db + 8 (v / 4) + 4 hi + v % 4.
-  const float i1 = 1.f / l[0], i2 = a.lambda / l[1];
+  const float i1 = 1.f / l;
   float ss = 0.f;
 #pragma unroll
   for (int db = 0; db < DB; ++db)
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
-      const float x = o[0][db][v] * i1 - o[1][db][v] * i2;
-      o[0][db][v] = x;
+      const float x = o[db][v] * i1 - x_s[(db * 16 + v) * 64 + lane];
+      o[db][v] = x;
       ss += x * x;   // padding columns hold zeros
     }
   ss += __shfl_xor(ss, 32, 64);
@@ -282,7 +283,7 @@ __global__ __launch_bounds__(256) void diff_attention_tiles_kernel(DiffAttnArgs 
       if (col < vdim) {   // value sizes are multiples of 8: four columns are there together
         union { __bf16 b[4]; uint2 u; } w;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) w.b[e] = (__bf16)(o[0][db][4 * v4 + e] * r);
+        for (int e = 0; e < 4; ++e) w.b[e] = (__bf16)(o[db][4 * v4 + e] * r);
         *(uint2*)(orow + col) = w.u;
       }
     }
@@ -297,11 +298,13 @@ bool diff_attention_tiles_takes(const DiffAttnArgs& a) {
 // rows of the tile (at most 32 of them), so that a block reads the keys and values of its kv
 // head once for all of them. A block owns one row, one kv head and one chunk of the context;
 // its four waves share every tile of 64 keys: wave w takes map w / 2 and the tile's keys
-// 32 (w % 2) .. + 31, with a running maximum, sum and output of its own. Every wave writes its
+// 32 (w % 2) .. + 31, with a running maximum, sum and output of its own. One buffer of LDS
+// (two barriers a tile, the next tile on its way in registers meanwhile), so that four
+// blocks fit a CU: what keeps the memory busy is the number of tiles under way. Every wave writes its
 // part of a record {m1, l1, m2, l2, acc1[vdim], acc2[vdim]} (one record per chunk and half),
 // and the merge kernel puts the records of a row and head together.
 template <int KS, int DB>
-__global__ __launch_bounds__(256) void diff_attention_heads_kernel(DiffAttnArgs a, int chunk,
+__global__ __launch_bounds__(256, 2) void diff_attention_heads_kernel(DiffAttnArgs a, int chunk,
                                                                    int n_chunks) {
   constexpr int DP = 16 * KS, KROW = 2 * DP + 8, VP = 32 * DB, VROW = VP + 8;
   constexpr int TILE = 64 * KROW + 64 * VROW;
@@ -331,7 +334,7 @@ __global__ __launch_bounds__(256) void diff_attention_heads_kernel(DiffAttnArgs 
   const unsigned short* vpool = (const unsigned short*)a.vpool;
   const int pos_last = last;   // (the name the tile macros use: no key beyond it is loaded)
 
-  for (int i = tid; i < 2 * TILE / 8; i += 256) ((u32x4*)lds)[i] = u32x4{0u, 0u, 0u, 0u};
+  for (int i = tid; i < TILE / 8; i += 256) ((u32x4*)lds)[i] = u32x4{0u, 0u, 0u, 0u};
 
   int k_key[KS], k_src[KS], k_dst[KS], v_key[DB], v_src[DB];
   bool k_ok[KS], v_ok[DB];
@@ -387,12 +390,13 @@ __global__ __launch_bounds__(256) void diff_attention_heads_kernel(DiffAttnArgs 
   __syncthreads();
   const int n_kt = (last - first) / 64 + 1;
   for (int kt = 0; kt < n_kt; ++kt) {
-    const int k0 = first + kt * 64, buf = kt & 1;
-    NINFER_DIFF_STORE_TILE(buf)
+    const int k0 = first + kt * 64;
+    if (kt > 0) __syncthreads();   // everyone has read the tile before: it may be written over
+    NINFER_DIFF_STORE_TILE(0)
     __syncthreads();
     if (kt + 1 < n_kt) NINFER_DIFF_LOAD_TILE(k0 + 64)
     if (k0 + 32 * kb > last) continue;   // none of this wave's keys is there
-    const unsigned short* ks_ = lds + buf * TILE;
+    const unsigned short* ks_ = lds;
     const unsigned short* vs_ = ks_ + 64 * KROW;
     f32x16 s;
 #pragma unroll
@@ -473,12 +477,13 @@ bool diff_attention_heads_takes(const DiffAttnArgs& a) {
   return diff_attention_tiles_takes(a) && a.max_qlen == 1 && a.Hq / a.Hkv <= 32;
 }
 
-// Chunks of the context (multiples of 64 keys) so that the launch has about two blocks a CU.
+// Chunks of the context (multiples of 64 keys) so that the launch has about four blocks a CU.
 void diff_attention_heads_plan(const DiffAttnArgs& a, int* chunk, int* n_chunks) {
   const int blocks = a.T * a.Hkv;
-  const int want = (2 * device_cu_count() + blocks - 1) / blocks;
+  const int want = (4 * device_cu_count() + blocks - 1) / blocks;
   int per = (a.max_kv_len + want - 1) / want;
-  per = ((per < 128 ? 128 : per) + 63) / 64 * 64;
+  // (at least 256 keys a chunk: every chunk leaves two records a head for the merge to read)
+  per = ((per < 256 ? 256 : per) + 63) / 64 * 64;
   *chunk = per;
   *n_chunks = (a.max_kv_len + per - 1) / per;
 }
@@ -486,7 +491,7 @@ void diff_attention_heads_plan(const DiffAttnArgs& a, int* chunk, int* n_chunks)
 template <int KS, int DB>
 static int launch_heads(const DiffAttnArgs& a, int chunk, int n_chunks, hipStream_t stream) {
   constexpr int DP = 16 * KS, VP = 32 * DB;
-  const size_t lds = 2 * (64 * (2 * DP + 8) + 64 * (VP + 8)) * sizeof(unsigned short);
+  const size_t lds = (64 * (2 * DP + 8) + 64 * (VP + 8)) * sizeof(unsigned short);
   auto kern = diff_attention_heads_kernel<KS, DB>;
   if (lds > 64 * 1024) {
     static bool raised = false;
@@ -526,8 +531,8 @@ int diff_attention_heads(const DiffAttnArgs& a, int chunk, int n_chunks, hipStre
 template <int KS, int DB>
 static int launch_tiles(const DiffAttnArgs& a, hipStream_t stream) {
   const int hpg = a.Hq / a.Hkv;
-  const int HB = hpg % 4 == 0 ? 4 : (hpg % 2 == 0 ? 2 : 1);
-  const int RT = 32 * (4 / HB);
+  const int HB = hpg % 2 == 0 ? 2 : 1;
+  const int RT = 32 * (2 / HB);
   constexpr int DP = 16 * KS, VP = 32 * DB;
   const size_t lds = 2 * (64 * (2 * DP + 8) + 64 * (VP + 8)) * sizeof(unsigned short);
   auto kern = diff_attention_tiles_kernel<KS, DB>;
