@@ -72,5 +72,49 @@ def config_straight():
     return cfg
 
 
+def random_config(seed):
+    """A seeded random configuration: head counts and groups of every kind, sizes in steps of
+    8 and others, widths and vocabularies that are no power of two, layers of every kind of
+    feed-forward in any order, with and without pair table, caps, temperature, loop."""
+    import random
+    rng = random.Random(seed)
+    width = rng.choice([40, 64, 72, 96, 100, 128, 136, 192])
+
+    def mixer():
+        kv = rng.choice([1, 2, 3])
+        dim = rng.choice([8, 12, 16, 24, 32, 40, 64, 80])
+        return _mixer(kv * rng.choice([1, 1, 2, 3, 4, 5]), kv, dim, rng.choice([8, 16, 20, 24, 40, 64, 96, 128]),
+                      diff=rng.choice([0.1, 0.35, 0.6, 0.8]), cap=rng.choice([None, 8.0, 30.0, 50.0]),
+                      temp=rng.choice([None, (0.3, 64), (0.5, 8), (1.0, 1), (0.2, 17)]))
+
+    def mlp():
+        kind = rng.choice(["none", "dense", "moe", "moe", "moe"])
+        if kind == "none":
+            return None
+        if kind == "dense":
+            return {"kind": "dense", "ff": rng.choice([24, 64, 100, 160])}
+        count = rng.choice([1, 2, 3, 4, 8])
+        per = rng.choice([1, 2, 3, 4, 6])
+        keep = rng.randint(1, count)
+        top = rng.randint(1, min(keep * per, 6))
+        return _moe(rng.choice([16, 24, 40, 64]), count * per, top,
+                    groups=None if count == 1 and rng.random() < 0.5 else (count, keep),
+                    shared=rng.choice([None, 16, 48, 72]))
+
+    n = rng.randint(1, 5)
+    cfg = {"architecture": "Sosepel", "vocab": rng.choice([97, 256, 333, 600]), "width": width,
+           "norm": {"eps": rng.choice([1e-6, 1e-5])}, "embedding": {"scale": rng.choice([0.5, 1.0, 3.0])},
+           "layers": [_layer(mixer(), mlp()) for _ in range(n)]}
+    if rng.random() < 0.7:
+        cfg["logit_softcap"] = rng.choice([5.0, 15.0, 30.0])
+    if rng.random() < 0.7:
+        cfg["embedding"]["bigram"] = {"buckets": rng.choice([1, 13, 509, 4099]),
+                                      "mul_prev": rng.choice([1, 127, 65537]), "mul_cur": rng.choice([1, 7, 31])}
+    if rng.random() < 0.7:
+        start = rng.randrange(n)
+        cfg["loop"] = {"start": start, "stop": rng.randint(start + 1, n), "times": rng.randint(1, 3)}
+    return cfg
+
+
 CASES = {"odd": (config_odd, 11), "even": (config_even, 22), "ones": (config_ones, 33),
          "straight": (config_straight, 44)}

@@ -368,8 +368,10 @@ def safe_prompt(w, cfg, n, seed, rel_margin=0.05):
         tries += 1
         if all(float(m[-1]) >= rel_margin for m in margins):
             toks.append(cand)
-        elif tries > 40 * n + 100:
-            raise RuntimeError("no prompt with clear routing found")
+        elif tries % (10 * n + 50) == 0:
+            rel_margin /= 2   # (many sparse layer runs: settle for less)
+            if rel_margin < 2e-3:
+                raise RuntimeError("no prompt with clear routing found")
     return toks
 
 
@@ -573,6 +575,31 @@ def test_decoding_from_a_captured_graph(case, dtype):
     for k in reqs:
         runner.close(slots[k])
     check_logits(case, dtype, {k: torch.cat(v) for k, v in got.items()}, "graph replay")
+
+
+@pytest.mark.parametrize("seed", list(range(9)))
+def test_random_configurations(seed, tmp_path):
+    """Configurations drawn at random (sizes, head counts, kinds and order of layers, what is
+    absent), in both precisions: whole, in portions and in a mixed batch."""
+    import ninfer_amd
+    from ninfer_amd import EngineOptions, load_model
+    raw = sosepel_cases.random_config(seed)
+    for dtype in ("float32", "bfloat16"):
+        d = str(tmp_path / dtype)
+        ninfer_amd.write_random_model(d, raw, 100 + seed, dtype=dtype, std=STD)
+        cfg, w = util.read_folder(d)
+        if dtype == "float32":
+            reqs = {f"q{i}": safe_prompt(w, cfg, n, 7 * seed + i) for i, n in enumerate([33, 1, 14, 50])}
+        ref = {k: plain_sosepel.forward(w, cfg, v) for k, v in reqs.items()}
+        case = {"name": f"random {seed}", "ref": {dtype: ref},
+                "noise": {dtype: {k: noise_of(cfg, w, v, ref[k]) for k, v in reqs.items()}}}
+        runner = load_model(d, EngineOptions(dtype=dtype, max_context=64, num_sequences=3, page_size=8,
+                                             num_pages=20, check_pages=True, poison_freed_pages=True))
+        for k, v in reqs.items():
+            check_logits(case, dtype, util.run_schedule(runner, util.schedule_whole(k, v)), "whole")
+            check_logits(case, dtype, util.run_schedule(runner, util.schedule_portions(k, v, seed=seed)), "portions")
+        check_logits(case, dtype, util.run_schedule(runner, util.schedule_mixed(reqs, seed=seed, max_live=3)), "mixed")
+        runner.release()
 
 
 def test_greedy_generation_through_the_scheduler(case):
