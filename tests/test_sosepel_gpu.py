@@ -2,7 +2,8 @@
 kernel, then whole models (four small configurations, in 32-bit and in bfloat16) layer by
 layer, whole, decoded token by token, in portions down to two tokens, in mixed batches with
 pages and state slots that are given back and used again, from a captured graph, generated
-greedily through the scheduler, and through the trace replay program. bfloat16 is compared
+greedily through the scheduler, through the command line and the trace replay program, and
+configurations drawn at random. bfloat16 is compared
 with the plain implementation on the bfloat16-rounded weights. Prompts are chosen so that no
 routing decision of the plain implementation is a close call."""
 import json
@@ -627,6 +628,34 @@ def test_greedy_generation_through_the_scheduler(case):
     eng.close()
     assert sum(len(x) for x in want) >= new
     assert [g[:len(x)] for g, x in zip(got, want)] == want
+
+
+def test_command_line(case):
+    """`ninfer <folder>` on a Sosepel folder: greedy from given and random prompts in 32-bit, the
+    first against the plain choice; sampling with the defaults from a captured graph in
+    bfloat16, the same seed the same tokens."""
+    if case["name"] != "even":
+        pytest.skip("one configuration is enough for the program")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    cfg, w = util.read_folder(case["dirs"]["float32"])
+    prompt = case["reqs"]["r2"][:9]
+    want = list(prompt)
+    for _ in range(4):
+        want.append(int(plain_sosepel.forward(w, cfg, want)[-1].argmax()))
+    run = lambda d, *more: subprocess.run(
+        [sys.executable, os.path.join(root, "bin", "ninfer"), d, "--prompt-ids", ",".join(map(str, prompt)),
+         "--max-context", "64", "--prefill-chunk", "8", *more], capture_output=True, text=True, timeout=300)
+    proc = run(case["dirs"]["float32"], "--random-prompts", "5,12", "--max-new", "4", "--temperature", "0",
+               "--dtype", "fp32", "--repeat-penalty", "1", "--eos-id", "-1")
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    lines = proc.stdout.strip().splitlines()
+    assert len(lines) == 3 and [int(x) for x in lines[0].split(",")] == want[len(prompt):]
+    outs = []
+    for _ in range(2):
+        proc = run(case["dirs"]["bfloat16"], "--max-new", "12", "--seed", "7", "--graph", "--eos-id", "-1")
+        assert proc.returncode == 0, proc.stderr[-2000:]
+        outs.append(proc.stdout.strip())
+    assert outs[0] == outs[1] and len(outs[0].split(",")) == 12
 
 
 def test_trace_replay_program(case, tmp_path):
