@@ -33,6 +33,8 @@ struct DiffAttnArgs {
   int max_qlen;             // host-side bounds that size launches
   int max_kv_len;
   int force_plain;
+  int single_rows;          // the first single_rows requests bring one row each: rows 0 .. single_rows - 1
+                            // (0 when the caller does not sort them)
   float scale;
   float cap;
   float t_coef;
@@ -44,7 +46,8 @@ struct DiffAttnArgs {
 
 int diff_attention_plain(const DiffAttnArgs& a, int chunk, int n_chunks, hipStream_t stream);
 bool diff_attention_tiles_takes(const DiffAttnArgs& a);
-int diff_attention_tiles(const DiffAttnArgs& a, hipStream_t stream);
+// (the requests before `first_seq` are left out: their single rows run as decode rows do)
+int diff_attention_tiles(const DiffAttnArgs& a, int first_seq, hipStream_t stream);
 // single rows with the heads of a kv head as the tile's rows: chunks, then the merge
 bool diff_attention_heads_takes(const DiffAttnArgs& a);
 void diff_attention_heads_plan(const DiffAttnArgs& a, int* chunk, int* n_chunks);

@@ -522,8 +522,28 @@ extern "C" int ninfer_diff_kv_write(const DiffAttnArgs* a, hipStream_t stream) {
   return 0;
 }
 
+// The single rows at the head of a step that also brings prompt portions, as a step of their
+// own (they run as decode rows do); T == 0: there are none, or the kernels for it do not take
+// the shape.
+static DiffAttnArgs diff_single_rows(const DiffAttnArgs& a) {
+  DiffAttnArgs s = a;
+  s.T = 0;
+  if (a.max_qlen > 1 && a.single_rows > 0 && a.single_rows < a.T && !a.force_plain &&
+      diff_attention_tiles_takes(a)) {
+    s.T = s.S = a.single_rows;
+    s.max_qlen = 1;
+    if (!diff_attention_heads_takes(s)) s.T = 0;
+  }
+  return s;
+}
+
 extern "C" long long ninfer_diff_attention_workspace_floats(const DiffAttnArgs* a) {
   int chunk, n;
+  const DiffAttnArgs single = diff_single_rows(*a);
+  if (single.T > 0) {
+    diff_attention_heads_plan(single, &chunk, &n);
+    return (long long)single.T * a->Hq * 2 * n * (4 + 2 * a->vdim);
+  }
   if (!a->force_plain && diff_attention_heads_takes(*a)) {
     diff_attention_heads_plan(*a, &chunk, &n);
     return (long long)a->T * a->Hq * 2 * n * (4 + 2 * a->vdim);
@@ -536,8 +556,16 @@ extern "C" int ninfer_diff_attention(const DiffAttnArgs* a, hipStream_t stream) 
   int rc = diff_check(*a, "diff_attention");
   if (rc) return rc;
   NINFER_REQUIRE(a->out && a->qkv && a->kpool && a->vpool, "diff_attention: null tensors");
-  if (a->max_qlen > 1 && !a->force_plain && diff_attention_tiles_takes(*a))
-    return diff_attention_tiles(*a, stream);
+  if (a->max_qlen > 1 && !a->force_plain && diff_attention_tiles_takes(*a)) {
+    const DiffAttnArgs single = diff_single_rows(*a);
+    if (single.T > 0) {
+      int chunk, n;
+      diff_attention_heads_plan(single, &chunk, &n);
+      rc = diff_attention_heads(single, chunk, n, stream);
+      if (rc) return rc;
+    }
+    return diff_attention_tiles(*a, single.T, stream);
+  }
   int chunk, n;
   if (!a->force_plain && diff_attention_heads_takes(*a)) {
     diff_attention_heads_plan(*a, &chunk, &n);

@@ -36,7 +36,8 @@ typedef __attribute__((address_space(3))) short4v lds_short4;
 constexpr float kLog2e = 1.44269504088896f;
 
 template <int KS, int DB>
-__global__ __launch_bounds__(256, 2) void diff_attention_tiles_kernel(DiffAttnArgs a, int HB) {
+__global__ __launch_bounds__(256, 2) void diff_attention_tiles_kernel(DiffAttnArgs a, int HB,
+                                                                      int first_seq) {
   constexpr int DP = 16 * KS, KROW = 2 * DP + 8, VP = 32 * DB, VROW = VP + 8;
   constexpr int TILE = 64 * KROW + 64 * VROW;   // elements of one buffer
   extern __shared__ __attribute__((aligned(16))) unsigned short lds[];
@@ -54,7 +55,7 @@ __global__ __launch_bounds__(256, 2) void diff_attention_tiles_kernel(DiffAttnAr
   int seq = -1, row0 = 0, n_rows = 0;
   {
     int idx = gridDim.x - 1 - blockIdx.x;   // the last row tiles of a request walk the most keys: first
-    for (int s = 0; s < a.S; ++s) {
+    for (int s = first_seq; s < a.S; ++s) {
       const int b = a.seq_row_start[s], e = a.seq_row_start[s + 1];
       const int nt = (e - b + RT - 1) / RT;
       if (idx < nt) {
@@ -529,7 +530,7 @@ int diff_attention_heads(const DiffAttnArgs& a, int chunk, int n_chunks, hipStre
 }
 
 template <int KS, int DB>
-static int launch_tiles(const DiffAttnArgs& a, hipStream_t stream) {
+static int launch_tiles(const DiffAttnArgs& a, int first_seq, hipStream_t stream) {
   const int hpg = a.Hq / a.Hkv;
   const int HB = hpg % 2 == 0 ? 2 : 1;
   const int RT = 32 * (2 / HB);
@@ -544,21 +545,22 @@ static int launch_tiles(const DiffAttnArgs& a, hipStream_t stream) {
       raised = true;
     }
   }
-  dim3 grid(a.T / RT + a.S, a.Hkv * (hpg / HB));
-  kern<<<grid, 256, lds, stream>>>(a, HB);
+  // (requests before first_seq bring one row each)
+  dim3 grid((a.T - first_seq) / RT + a.S - first_seq, a.Hkv * (hpg / HB));
+  kern<<<grid, 256, lds, stream>>>(a, HB, first_seq);
   NINFER_LAUNCH_CHECK();
   return 0;
 }
 
-int diff_attention_tiles(const DiffAttnArgs& a, hipStream_t stream) {
+int diff_attention_tiles(const DiffAttnArgs& a, int first_seq, hipStream_t stream) {
   const int db = (a.vdim + 31) / 32;
   const int ks = a.dim <= 32 ? 2 : a.dim <= 48 ? 3 : a.dim <= 64 ? 4 : a.dim <= 96 ? 6 : 8;
 #define NINFER_DIFF_TILES(KS_)                                   \
   switch (db) {                                                  \
-    case 1: return launch_tiles<KS_, 1>(a, stream);              \
-    case 2: return launch_tiles<KS_, 2>(a, stream);              \
-    case 3: return launch_tiles<KS_, 3>(a, stream);              \
-    default: return launch_tiles<KS_, 4>(a, stream);             \
+    case 1: return launch_tiles<KS_, 1>(a, first_seq, stream);              \
+    case 2: return launch_tiles<KS_, 2>(a, first_seq, stream);              \
+    case 3: return launch_tiles<KS_, 3>(a, first_seq, stream);              \
+    default: return launch_tiles<KS_, 4>(a, first_seq, stream);             \
   }
   switch (ks) {
     case 2: NINFER_DIFF_TILES(2)

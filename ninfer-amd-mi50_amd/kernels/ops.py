@@ -119,7 +119,8 @@ class _DiffAttnArgs(ctypes.Structure):
                 ("Hq", ctypes.c_int), ("Hkv", ctypes.c_int), ("dim", ctypes.c_int),
                 ("vdim", ctypes.c_int), ("page_size", ctypes.c_int), ("dtype", ctypes.c_int),
                 ("max_qlen", ctypes.c_int), ("max_kv_len", ctypes.c_int),
-                ("force_plain", ctypes.c_int), ("scale", ctypes.c_float), ("cap", ctypes.c_float),
+                ("force_plain", ctypes.c_int), ("single_rows", ctypes.c_int),
+                ("scale", ctypes.c_float), ("cap", ctypes.c_float),
                 ("t_coef", ctypes.c_float), ("t_every", ctypes.c_int), ("lam", ctypes.c_float),
                 ("eps", ctypes.c_float), ("out_scale", ctypes.c_float)]
 
@@ -1220,6 +1221,7 @@ class HipOps:
         a.Hq, a.Hkv, a.dim, a.vdim, a.page_size = heads, kv_heads, dim, vdim, page_size
         a.dtype, a.max_qlen, a.max_kv_len = _DT[qkv.dtype], ctx.max_qlen, ctx.max_kv_len
         a.force_plain = 1 if self.force_generic else 0
+        a.single_rows = int(getattr(ctx, "single_rows", 0))
         a.scale, a.cap, a.t_coef, a.t_every = scale, cap, temp_coef, int(temp_every)
         a.lam, a.eps, a.out_scale = lam, eps, out_scale
         if write_kv:
