@@ -530,15 +530,15 @@ def sosepel_config(z: dict) -> dict:
     """A dense first layer, then sparse ones; the layers between the first and the last run
     twice, each run with a cache of its own."""
     mixer = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["vdim"],
-             "diff": 0.6, "scale": z["dim"] ** -0.5, "softcap": 50.0, "q_temp": {"coef": 0.3, "every": 64}}
+             "diff": 0.5, "scale": z["dim"] ** -0.5, "softcap": 30.0, "q_temp": {"coef": 0.25, "every": 128}}
     moe = {"kind": "moe", "expert": {"ff": z["expert_ff"]}, "shared": {"ff": z["shared_ff"]},
            "router": {"experts": z["experts"], "top": z["top"],
                       "groups": {"count": z["groups"][0], "keep": z["groups"][1]}}}
     layers = [{"type": "attention", "mixer": mixer, "mlp": {"kind": "dense", "ff": z["ff"]}}]
     layers += [{"type": "attention", "mixer": mixer, "mlp": moe} for _ in range(z["layers"] - 1)]
     return {"architecture": "Sosepel", "vocab": z["vocab"], "width": z["width"], "norm": {"eps": 1e-6},
-            "logit_softcap": 15.0, "embedding": {"scale": 0.5, "bigram": {"buckets": 65521, "mul_prev": 127,
-                                                                         "mul_cur": 7}},
+            "logit_softcap": 20.0, "embedding": {"scale": 1.0, "bigram": {"buckets": 65521, "mul_prev": 31,
+                                                                         "mul_cur": 3}},
             "layers": layers, "loop": {"start": 1, "stop": z["layers"] - 1, "times": 2}}
 
 

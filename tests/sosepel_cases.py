@@ -84,8 +84,8 @@ def random_config(seed):
         kv = rng.choice([1, 2, 3])
         dim = rng.choice([8, 12, 16, 24, 32, 40, 64, 80])
         return _mixer(kv * rng.choice([1, 1, 2, 3, 4, 5]), kv, dim, rng.choice([8, 16, 20, 24, 40, 64, 96, 128]),
-                      diff=rng.choice([0.1, 0.35, 0.6, 0.8]), cap=rng.choice([None, 8.0, 30.0, 50.0]),
-                      temp=rng.choice([None, (0.3, 64), (0.5, 8), (1.0, 1), (0.2, 17)]))
+                      diff=rng.choice([0.1, 0.35, 0.6, 0.8]), cap=rng.choice([None, 8.0, 30.0, 40.0]),
+                      temp=rng.choice([None, (0.3, 32), (0.5, 8), (1.0, 1), (0.2, 17)]))
 
     def mlp():
         kind = rng.choice(["none", "dense", "moe", "moe", "moe"])
@@ -103,13 +103,13 @@ def random_config(seed):
 
     n = rng.randint(1, 5)
     cfg = {"architecture": "Sosepel", "vocab": rng.choice([97, 256, 333, 600]), "width": width,
-           "norm": {"eps": rng.choice([1e-6, 1e-5])}, "embedding": {"scale": rng.choice([0.5, 1.0, 3.0])},
+           "norm": {"eps": rng.choice([1e-6, 1e-5])}, "embedding": {"scale": rng.choice([0.75, 1.0, 3.0])},
            "layers": [_layer(mixer(), mlp()) for _ in range(n)]}
     if rng.random() < 0.7:
-        cfg["logit_softcap"] = rng.choice([5.0, 15.0, 30.0])
+        cfg["logit_softcap"] = rng.choice([5.0, 12.0, 30.0])
     if rng.random() < 0.7:
-        cfg["embedding"]["bigram"] = {"buckets": rng.choice([1, 13, 509, 4099]),
-                                      "mul_prev": rng.choice([1, 127, 65537]), "mul_cur": rng.choice([1, 7, 31])}
+        cfg["embedding"]["bigram"] = {"buckets": rng.choice([1, 13, 521, 4099]),
+                                      "mul_prev": rng.choice([1, 131, 65537]), "mul_cur": rng.choice([1, 5, 31])}
     if rng.random() < 0.7:
         start = rng.randrange(n)
         cfg["loop"] = {"start": start, "stop": rng.randint(start + 1, n), "times": rng.randint(1, 3)}
